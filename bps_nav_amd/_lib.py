@@ -80,6 +80,10 @@ def lib():
             L.bpsx_get_state.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(State)]
             L.bpsx_check_errors.argtypes = [C.c_void_p]
             L.bpsx_get_counters.argtypes = [C.c_void_p, C.c_void_p]
+            L.bpsx_set_profiling.argtypes = [C.c_void_p, C.c_int]
+            L.bpsx_get_kernel_times.argtypes = [C.c_void_p, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]
+            L.bpsx_kernel_name.argtypes = [C.c_uint32]
+            L.bpsx_kernel_name.restype = C.c_char_p
             L.bpsx_snap_points.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p]
             L.bpsx_try_steps.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_uint32, C.c_void_p, C.c_void_p]

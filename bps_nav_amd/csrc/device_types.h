@@ -1,0 +1,136 @@
+// Layout of the navmesh and agent data in HBM, shared by the host uploader and the kernels.
+//
+// Polygons are stored as one 128-byte record each (one L2 cache line on gfx950), so a walk
+// that hops from polygon to polygon costs exactly one line per hop: vertices, neighbours,
+// filter result and the handle of the height mesh travel together.  Everything an agent
+// gathers per step is indexed by (scene polygon base + polygon index).
+#pragma once
+#include <cstdint>
+
+namespace bpsx {
+
+constexpr int kNvp = 6;
+constexpr uint32_t kInvalidPoly = 0xffffffffu;
+
+// Detour buffer limits that are part of the reference's observable behaviour.
+constexpr int kMaxNodes = 2048;     // dtNavMeshQuery::init(nav, 2048), PathFinder.cpp:247
+constexpr int kMaxPath = 256;       // MAX_POLYS, PathFinder.cpp:499, 546
+constexpr int kTinyNodes = 64;      // m_tinyNodePool, DetourNavMeshQuery.cpp:191
+constexpr int kMoveQueue = 48;      // MAX_STACK, DetourNavMeshQuery.cpp:2039
+
+struct alignas(128) PolyRec {
+  float v[kNvp][3];        // vertex positions, polygon order
+  uint16_t nei[kNvp];      // raw Detour neis: 0 wall, idx+1 internal, 0x8000|dir tile border
+  uint16_t walk[kNvp];     // idx+1 of the neighbour across edge j if it passes the query
+                           // filter (PathFinder.cpp:239-243), else 0
+  uint16_t flags;          // polygon flags after zero-area disabling (PathFinder.cpp:307-328)
+  uint8_t nv;              // vertex count
+  uint8_t type;            // 0 ground, 1 off-mesh connection
+  uint32_t tri_base;       // first detail triangle, index into the global triangle array
+  uint32_t dvert_base;     // first extra detail vertex, index into the global array
+  uint8_t tri_count;
+  uint8_t dvert_count;
+  uint16_t pad0;
+  uint32_t island;         // connected component id (IslandSystem, PathFinder.cpp:53-170)
+  float area_cum;          // inclusive prefix sum of walkable fan areas (sampling)
+  uint32_t pad1[2];
+};
+static_assert(sizeof(PolyRec) == 128, "PolyRec must be one cache line");
+
+struct BVNodeDev {  // dtBVNode
+  uint16_t bmin[3], bmax[3];
+  int32_t i;
+};
+static_assert(sizeof(BVNodeDev) == 16, "BV node");
+
+struct SceneDev {
+  uint32_t poly_base, poly_count;
+  uint32_t bv_base, bv_count;
+  uint32_t ep_base, ep_count;       // rows of 10 floats in the episode array
+  uint32_t ref_base;                // salt and tile bits of every polygon ref of the scene
+  uint32_t poly_mask;               // (1 << polyBits) - 1
+  float orig[3], tile_w, tile_h;    // dtNavMeshParams
+  int32_t tx, ty;                   // tile grid location
+  float bmin[3], bmax[3];           // tile bounds
+  float qfac;                       // bvQuantFactor
+  float climb;                      // walkableClimb
+  float area_total;
+  uint32_t pad[3];
+};
+
+// ---- per-agent state, structure of arrays over all agents of the simulator
+struct AgentArrays {
+  float* pos;         // [N][3]
+  float* rot;         // [N][4] x,y,z,w
+  float* goal;        // [N][3]
+  float* nav_xyz;     // [N][3] navmeshPosition_.xyz
+  uint32_t* nav_ref;  // [N]    navmeshPosition_.polyId
+  float* goal_xyz;    // [N][3] navmeshGoal_.xyz
+  uint32_t* goal_ref; // [N]
+  float* prev_pos;    // [N][3]
+  float* info_prev;   // [N] InfoFunctor::prev_distance_to_goal_
+  float* cum;         // [N]
+  float* init;        // [N]
+  float* rew_prev;    // [N] RewardFunctor::prev_distance_to_goal_
+  uint32_t* step;     // [N]
+  uint32_t* scene;    // [N]
+  uint32_t* episode;  // [N]
+  uint32_t* nresets;  // [N]
+  uint32_t* flags;    // [N] transient per-step bits, see kAgent*
+  float* geo;         // [N] result slot of the geodesic kernel
+  // outputs
+  float* rewards;     // [N]
+  uint8_t* masks;     // [N]
+  float* infos;       // [N][3]
+  float* polars;      // [N][2]
+};
+constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentNeedGeo = 4u, kAgentSkip = 8u;
+
+struct NavData {
+  const PolyRec* polys;
+  const BVNodeDev* bv;
+  const uint8_t* dtris;    // [.][4]
+  const float* dverts;     // [.][3]
+  const SceneDev* scenes;
+  const float* episodes;   // [.][10]
+};
+
+// A* node of the per-slot pool (dtNode, DetourNode.h:36-45): 32 bytes.
+struct ANode {
+  float pos[3];
+  float cost;
+  float total;
+  uint32_t pidx;   // 1-based parent node index, 0 = none
+  uint32_t flags;  // 1 open, 2 closed
+  uint32_t id;     // polygon index within the scene
+};
+static_assert(sizeof(ANode) == 32, "ANode");
+
+struct HeapEntry {
+  float total;
+  uint32_t node;
+};
+
+// Scratch of one A* slot in HBM.
+struct alignas(128) GeoSlot {
+  ANode nodes[kMaxNodes];
+  HeapEntry heap_spill[kMaxNodes];   // heap entries beyond the LDS-resident top
+  uint16_t next[kMaxNodes];          // hash chains
+  uint32_t corridor[kMaxPath];
+  float portals[kMaxPath][6];        // left xyz, right xyz of corridor portal i -> i+1
+};
+
+struct GeoQuery {
+  float a[3];
+  uint32_t a_ref;
+  float b[3];
+  uint32_t b_ref;
+  uint32_t scene;
+  uint32_t out;   // index into the result array
+};
+
+enum Counter {
+  kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands
+};
+
+}  // namespace bpsx

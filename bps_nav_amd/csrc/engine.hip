@@ -1,0 +1,486 @@
+// Host side of libbpsx: the C ABI declared in include/bpsx.h, device memory ownership and
+// kernel sequencing.  The counterpart of RolloutGenerator / EnvironmentGroup
+// (simulator.cpp:1180-1330, 1332-1700) without worker threads: a step is a short chain of
+// kernels on the caller's HIP stream.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/bpsx.h"
+#include "errors.h"
+#include "kernels.h"
+#include "navmesh_host.h"
+
+using namespace bpsx;
+
+#define HIP_TRY(expr)                                                                            \
+  do {                                                                                           \
+    hipError_t e_ = (expr);                                                                      \
+    if (e_ != hipSuccess) return fail(BPSX_E_HIP, std::string(#expr) + ": " + hipGetErrorString(e_)); \
+  } while (0)
+
+namespace {
+
+const char* const kKernelNames[BPSX_NUM_KERNELS] = {"step_move", "geodesic_step", "step_finish",
+                                                    "reset_snap", "geodesic_reset", "reset_finish"};
+
+struct Group {
+  StepQueues Q{};
+  int64_t* d_actions = nullptr;
+  int64_t* h_actions = nullptr;  // pinned staging for host-side action arrays
+  hipEvent_t done = nullptr;
+  hipEvent_t ev[kStepEvents] = {};
+  bool in_flight = false;
+  bool profiled = false;
+};
+
+template <class T>
+int dev_alloc(T** p, size_t count) {
+  HIP_TRY(hipMalloc((void**)p, std::max<size_t>(count, 1) * sizeof(T)));
+  HIP_TRY(hipMemset(*p, 0, std::max<size_t>(count, 1) * sizeof(T)));
+  return BPSX_OK;
+}
+
+}  // namespace
+
+struct bpsx_sim {
+  bpsx_config cfg{};
+  std::vector<HostScene> scenes;
+  bool finalized = false;
+  uint32_t num_groups = 1, envs_per_group = 0;
+  // navmesh arrays
+  PolyRec* d_polys = nullptr;
+  BVNodeDev* d_bv = nullptr;
+  uint8_t* d_dtris = nullptr;
+  float* d_dverts = nullptr;
+  SceneDev* d_scenes = nullptr;
+  float* d_episodes = nullptr;
+  NavData nav{};
+  AgentArrays A{};
+  std::vector<void*> owned;  // every device allocation, for destroy
+  std::vector<Group> groups;
+  GeoSlot* d_slots = nullptr;
+  uint32_t geo_blocks = 0;
+  uint32_t* d_error = nullptr;
+  uint64_t* d_counters = nullptr;
+  float turn_left[4], turn_right[4];
+  // profiling
+  bool profiling = false;
+  double kernel_ms[BPSX_NUM_KERNELS] = {};
+  uint64_t profiled_steps = 0;
+  // scratch for the batched query entry points
+  void* d_batch = nullptr;
+  size_t batch_bytes = 0;
+  uint32_t* d_batch_counts = nullptr;
+
+  template <class T>
+  int alloc(T** p, size_t count) {
+    const int rc = dev_alloc(p, count);
+    if (rc == BPSX_OK) owned.push_back((void*)*p);
+    return rc;
+  }
+  StepParams params(uint32_t group) const {
+    StepParams P{};
+    P.n = envs_per_group;
+    P.base = group * envs_per_group;
+    P.max_steps = (float)(cfg.max_steps ? cfg.max_steps : BPSX_MAX_STEPS);
+    P.reset_mode = cfg.reset_mode;
+    P.seed = cfg.seed;
+    memcpy(P.turn_left, turn_left, 16);
+    memcpy(P.turn_right, turn_right, 16);
+    P.error_flag = d_error;
+    P.counters = d_counters;
+    return P;
+  }
+};
+
+extern "C" {
+
+int bpsx_create(const bpsx_config* cfg, bpsx_sim** out) {
+  if (!cfg || !out) return fail(BPSX_E_INVAL, "create: null argument");
+  if (!cfg->num_environments || !cfg->num_active_scenes) return fail(BPSX_E_INVAL, "create: zero environments or scenes");
+  const uint32_t groups = cfg->double_buffered ? 2 : 1;
+  if (cfg->num_environments % cfg->num_active_scenes != 0)
+    return fail(BPSX_E_INVAL, "create: num_environments is not a multiple of num_active_scenes");
+  if (cfg->num_active_scenes % groups != 0)
+    return fail(BPSX_E_INVAL, "create: num_active_scenes is not a multiple of the number of groups");
+  if (cfg->reset_mode > BPSX_RESET_SAMPLED) return fail(BPSX_E_INVAL, "create: unknown reset_mode");
+  int ndev = 0;
+  HIP_TRY(hipGetDeviceCount(&ndev));
+  if (cfg->gpu_id < 0 || cfg->gpu_id >= ndev) return fail(BPSX_E_INVAL, "create: gpu_id out of range");
+  bpsx_sim* s = new bpsx_sim();
+  s->cfg = *cfg;
+  s->num_groups = groups;
+  s->envs_per_group = cfg->num_environments / groups;
+  // glm::angleAxis(+-glm::radians(10.f), (0,1,0)) evaluated with the host libm, as the
+  // reference's static initialisers do (simulator.cpp:52-60)
+  const float a = BPSX_TURN_DEGREES * 0.01745329251994329576923690768489f;
+  s->turn_left[0] = 0; s->turn_left[1] = sinf(a * 0.5f); s->turn_left[2] = 0; s->turn_left[3] = cosf(a * 0.5f);
+  s->turn_right[0] = 0; s->turn_right[1] = sinf(-a * 0.5f); s->turn_right[2] = 0; s->turn_right[3] = cosf(-a * 0.5f);
+  *out = s;
+  return BPSX_OK;
+}
+
+int bpsx_add_scene(bpsx_sim* sim, const void* navmesh_bytes, size_t navmesh_size, const float* episodes,
+                   uint32_t num_episodes) {
+  if (!sim || !navmesh_bytes) return fail(BPSX_E_INVAL, "add_scene: null argument");
+  if (sim->finalized) return fail(BPSX_E_STATE, "add_scene: simulator already finalized");
+  if (sim->cfg.reset_mode == BPSX_RESET_EPISODES && (!episodes || !num_episodes))
+    return fail(BPSX_E_INVAL, "add_scene: episode-table reset needs at least one episode");
+  HostScene hs;
+  const int rc = parse_navmesh((const uint8_t*)navmesh_bytes, navmesh_size, &hs);
+  if (rc) return rc;
+  if (episodes && num_episodes) hs.episodes.assign(episodes, episodes + (size_t)num_episodes * 10);
+  hs.dev.ep_count = num_episodes;
+  sim->scenes.push_back(std::move(hs));
+  return BPSX_OK;
+}
+
+int bpsx_finalize(bpsx_sim* sim) {
+  if (!sim) return fail(BPSX_E_INVAL, "finalize: null simulator");
+  if (sim->finalized) return fail(BPSX_E_STATE, "finalize: called twice");
+  if (sim->scenes.size() != sim->cfg.num_active_scenes)
+    return fail(BPSX_E_INVAL, "finalize: number of scenes added differs from num_active_scenes");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  // ---- concatenate scenes
+  size_t npoly = 0, nbv = 0, ntri = 0, ndv = 0, nep = 0;
+  for (auto& s : sim->scenes) {
+    s.dev.poly_base = (uint32_t)npoly; s.dev.bv_base = (uint32_t)nbv; s.dev.ep_base = (uint32_t)nep;
+    for (auto& p : s.polys) { p.tri_base += (uint32_t)ntri; p.dvert_base += (uint32_t)ndv; }
+    npoly += s.polys.size(); nbv += s.bv.size(); ntri += s.dtris.size() / 4; ndv += s.dverts.size() / 3;
+    nep += s.episodes.size() / 10;
+  }
+  if (npoly > 0xfffffff0ull || ntri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
+  int rc;
+  if ((rc = sim->alloc(&sim->d_polys, npoly))) return rc;
+  if ((rc = sim->alloc(&sim->d_bv, nbv))) return rc;
+  if ((rc = sim->alloc(&sim->d_dtris, ntri * 4))) return rc;
+  if ((rc = sim->alloc(&sim->d_dverts, ndv * 3))) return rc;
+  if ((rc = sim->alloc(&sim->d_scenes, sim->scenes.size()))) return rc;
+  if ((rc = sim->alloc(&sim->d_episodes, nep * 10))) return rc;
+  std::vector<SceneDev> sd;
+  for (auto& s : sim->scenes) {
+    HIP_TRY(hipMemcpy(sim->d_polys + s.dev.poly_base, s.polys.data(), s.polys.size() * sizeof(PolyRec), hipMemcpyHostToDevice));
+    if (!s.bv.empty())
+      HIP_TRY(hipMemcpy(sim->d_bv + s.dev.bv_base, s.bv.data(), s.bv.size() * sizeof(BVNodeDev), hipMemcpyHostToDevice));
+    sd.push_back(s.dev);
+  }
+  // detail arrays and episodes are copied with running offsets
+  {
+    size_t toff = 0, voff = 0, eoff = 0;
+    for (auto& s : sim->scenes) {
+      if (!s.dtris.empty()) HIP_TRY(hipMemcpy(sim->d_dtris + toff, s.dtris.data(), s.dtris.size(), hipMemcpyHostToDevice));
+      if (!s.dverts.empty()) HIP_TRY(hipMemcpy(sim->d_dverts + voff, s.dverts.data(), s.dverts.size() * 4, hipMemcpyHostToDevice));
+      if (!s.episodes.empty()) HIP_TRY(hipMemcpy(sim->d_episodes + eoff, s.episodes.data(), s.episodes.size() * 4, hipMemcpyHostToDevice));
+      toff += s.dtris.size(); voff += s.dverts.size(); eoff += s.episodes.size();
+    }
+  }
+  HIP_TRY(hipMemcpy(sim->d_scenes, sd.data(), sd.size() * sizeof(SceneDev), hipMemcpyHostToDevice));
+  sim->nav = NavData{sim->d_polys, sim->d_bv, sim->d_dtris, sim->d_dverts, sim->d_scenes, sim->d_episodes};
+
+  // ---- agent state
+  const size_t N = sim->cfg.num_environments;
+  AgentArrays& A = sim->A;
+  if ((rc = sim->alloc(&A.pos, N * 3)) || (rc = sim->alloc(&A.rot, N * 4)) || (rc = sim->alloc(&A.goal, N * 3)) ||
+      (rc = sim->alloc(&A.nav_xyz, N * 3)) || (rc = sim->alloc(&A.nav_ref, N)) || (rc = sim->alloc(&A.goal_xyz, N * 3)) ||
+      (rc = sim->alloc(&A.goal_ref, N)) || (rc = sim->alloc(&A.prev_pos, N * 3)) || (rc = sim->alloc(&A.info_prev, N)) ||
+      (rc = sim->alloc(&A.cum, N)) || (rc = sim->alloc(&A.init, N)) || (rc = sim->alloc(&A.rew_prev, N)) ||
+      (rc = sim->alloc(&A.step, N)) || (rc = sim->alloc(&A.scene, N)) || (rc = sim->alloc(&A.episode, N)) ||
+      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.geo, N)) ||
+      (rc = sim->alloc(&A.rewards, N)) || (rc = sim->alloc(&A.masks, N)) || (rc = sim->alloc(&A.infos, N * 3)) ||
+      (rc = sim->alloc(&A.polars, N * 2)))
+    return rc;
+  {
+    // env -> scene: contiguous blocks of N / scenes (simulator.cpp:1205-1221, 1578-1592)
+    std::vector<uint32_t> scene(N);
+    const size_t per = N / sim->cfg.num_active_scenes;
+    for (size_t i = 0; i < N; ++i) scene[i] = (uint32_t)(i / per);
+    HIP_TRY(hipMemcpy(A.scene, scene.data(), N * 4, hipMemcpyHostToDevice));
+    std::vector<float> rot(N * 4, 0.f);
+    for (size_t i = 0; i < N; ++i) rot[i * 4 + 3] = 1.f;
+    HIP_TRY(hipMemcpy(A.rot, rot.data(), N * 16, hipMemcpyHostToDevice));
+  }
+  if ((rc = sim->alloc(&sim->d_error, 1)) || (rc = sim->alloc(&sim->d_counters, BPSX_NUM_COUNTERS))) return rc;
+  if ((rc = sim->alloc(&sim->d_batch_counts, 2))) return rc;
+
+  // ---- A* slots: a fixed pool sized by the device, not by the agent count
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, sim->cfg.gpu_id));
+  uint32_t per_cu = 12;
+  if (const char* e = getenv("BPSX_GEO_BLOCKS_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e));
+  const uint32_t gpw = 64 / kGeoGroup;
+  uint32_t blocks = (uint32_t)prop.multiProcessorCount * per_cu;
+  const uint32_t needed = (sim->envs_per_group + gpw - 1) / gpw;
+  if (blocks > needed) blocks = needed;
+  sim->geo_blocks = std::max(1u, blocks);
+  if ((rc = sim->alloc(&sim->d_slots, (size_t)sim->geo_blocks * gpw))) return rc;
+
+  // ---- per-group queues
+  sim->groups.resize(sim->num_groups);
+  const size_t n = sim->envs_per_group;
+  for (auto& g : sim->groups) {
+    if ((rc = sim->alloc(&g.Q.counts, 8)) || (rc = sim->alloc(&g.Q.step_queries, n)) ||
+        (rc = sim->alloc(&g.Q.reset_queries, n)) || (rc = sim->alloc(&g.Q.reset_list, n)) ||
+        (rc = sim->alloc(&g.d_actions, n)))
+      return rc;
+    HIP_TRY(hipHostMalloc((void**)&g.h_actions, n * sizeof(int64_t), hipHostMallocDefault));
+    HIP_TRY(hipEventCreateWithFlags(&g.done, hipEventDisableTiming));
+    for (auto& e : g.ev) HIP_TRY(hipEventCreate(&e));
+  }
+  sim->finalized = true;
+  return BPSX_OK;
+}
+
+void bpsx_destroy(bpsx_sim* sim) {
+  if (!sim) return;
+  if (sim->finalized) {
+    (void)hipSetDevice(sim->cfg.gpu_id);
+    (void)hipDeviceSynchronize();
+  }
+  for (auto& g : sim->groups) {
+    if (g.h_actions) (void)hipHostFree(g.h_actions);
+    if (g.done) (void)hipEventDestroy(g.done);
+    for (auto& e : g.ev)
+      if (e) (void)hipEventDestroy(e);
+  }
+  for (void* p : sim->owned) (void)hipFree(p);
+  if (sim->d_batch) (void)hipFree(sim->d_batch);
+  delete sim;
+}
+
+int bpsx_num_groups(const bpsx_sim* sim, uint32_t* out) {
+  if (!sim || !out) return fail(BPSX_E_INVAL, "num_groups: null argument");
+  *out = sim->num_groups;
+  return BPSX_OK;
+}
+
+static int check_group(bpsx_sim* sim, uint32_t group, const char* what) {
+  if (!sim) return fail(BPSX_E_INVAL, std::string(what) + ": null simulator");
+  if (!sim->finalized) return fail(BPSX_E_STATE, std::string(what) + ": simulator not finalized");
+  if (group >= sim->num_groups) return fail(BPSX_E_INVAL, std::string(what) + ": group out of range");
+  return BPSX_OK;
+}
+
+int bpsx_reset(bpsx_sim* sim, uint32_t group, void* hip_stream) {
+  int rc = check_group(sim, group, "reset");
+  if (rc) return rc;
+  Group& g = sim->groups[group];
+  if (g.in_flight) return fail(BPSX_E_STATE, "reset: a step of this group is still in flight");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  hipStream_t st = (hipStream_t)hip_stream;
+  launch_reset(sim->nav, sim->A, g.Q, sim->params(group), sim->d_slots, sim->geo_blocks, st);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipStreamSynchronize(st));
+  return BPSX_OK;
+}
+
+int bpsx_step_start(bpsx_sim* sim, uint32_t group, const int64_t* actions, int actions_on_device, void* hip_stream) {
+  int rc = check_group(sim, group, "step_start");
+  if (rc) return rc;
+  if (!actions) return fail(BPSX_E_INVAL, "step_start: null actions");
+  Group& g = sim->groups[group];
+  // the reference aborts with "Not done with previous simulation" (simulator.cpp:1659-1662)
+  for (auto& og : sim->groups)
+    if (og.in_flight) return fail(BPSX_E_STATE, "step_start: previous step not finished (call step_end first)");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  hipStream_t st = (hipStream_t)hip_stream;
+  const int64_t* d_act = actions;
+  if (!actions_on_device) {
+    memcpy(g.h_actions, actions, (size_t)sim->envs_per_group * sizeof(int64_t));
+    HIP_TRY(hipMemcpyAsync(g.d_actions, g.h_actions, (size_t)sim->envs_per_group * sizeof(int64_t), hipMemcpyHostToDevice, st));
+    d_act = g.d_actions;
+  }
+  g.profiled = sim->profiling;
+  launch_step(sim->nav, sim->A, g.Q, sim->params(group), d_act, sim->d_slots, sim->geo_blocks, st,
+              g.profiled ? g.ev : nullptr);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipEventRecord(g.done, st));
+  g.in_flight = true;
+  return BPSX_OK;
+}
+
+int bpsx_step_end(bpsx_sim* sim, uint32_t group) {
+  int rc = check_group(sim, group, "step_end");
+  if (rc) return rc;
+  Group& g = sim->groups[group];
+  // the reference aborts with "Simulation already done" / group mismatch (simulator.cpp:1679-1689)
+  if (!g.in_flight) return fail(BPSX_E_STATE, "step_end: no step in flight for this group");
+  HIP_TRY(hipEventSynchronize(g.done));
+  g.in_flight = false;
+  if (g.profiled) {
+    for (int k = 0; k < BPSX_NUM_KERNELS; ++k) {
+      float ms = 0;
+      HIP_TRY(hipEventElapsedTime(&ms, g.ev[k], g.ev[k + 1]));
+      sim->kernel_ms[k] += ms;
+    }
+    sim->profiled_steps++;
+  }
+  return BPSX_OK;
+}
+
+int bpsx_get_outputs(bpsx_sim* sim, uint32_t group, bpsx_outputs* out) {
+  int rc = check_group(sim, group, "get_outputs");
+  if (rc) return rc;
+  if (!out) return fail(BPSX_E_INVAL, "get_outputs: null argument");
+  const size_t b = (size_t)group * sim->envs_per_group;
+  out->rewards = sim->A.rewards + b;
+  out->masks = sim->A.masks + b;
+  out->infos = sim->A.infos + b * 3;
+  out->polars = sim->A.polars + b * 2;
+  out->n = sim->envs_per_group;
+  return BPSX_OK;
+}
+
+int bpsx_get_state(bpsx_sim* sim, uint32_t group, bpsx_state* out) {
+  int rc = check_group(sim, group, "get_state");
+  if (rc) return rc;
+  if (!out) return fail(BPSX_E_INVAL, "get_state: null argument");
+  const size_t b = (size_t)group * sim->envs_per_group;
+  out->position = sim->A.pos + b * 3;
+  out->rotation = sim->A.rot + b * 4;
+  out->goal = sim->A.goal + b * 3;
+  out->poly_ref = sim->A.nav_ref + b;
+  out->goal_ref = sim->A.goal_ref + b;
+  out->step = sim->A.step + b;
+  out->episode = sim->A.episode + b;
+  out->num_resets = sim->A.nresets + b;
+  out->n = sim->envs_per_group;
+  return BPSX_OK;
+}
+
+int bpsx_check_errors(bpsx_sim* sim) {
+  if (!sim || !sim->finalized) return fail(BPSX_E_STATE, "check_errors: simulator not finalized");
+  uint32_t f = 0;
+  HIP_TRY(hipMemcpy(&f, sim->d_error, 4, hipMemcpyDeviceToHost));
+  if (f) return fail(BPSX_E_ACTION, "an action id outside 0..3 was passed to step");
+  return BPSX_OK;
+}
+
+int bpsx_get_counters(bpsx_sim* sim, uint64_t* out) {
+  if (!sim || !sim->finalized || !out) return fail(BPSX_E_STATE, "get_counters: simulator not finalized");
+  HIP_TRY(hipMemcpy(out, sim->d_counters, BPSX_NUM_COUNTERS * 8, hipMemcpyDeviceToHost));
+  return BPSX_OK;
+}
+
+int bpsx_set_profiling(bpsx_sim* sim, int enabled) {
+  if (!sim) return fail(BPSX_E_INVAL, "set_profiling: null simulator");
+  sim->profiling = enabled != 0;
+  if (enabled) {
+    memset(sim->kernel_ms, 0, sizeof(sim->kernel_ms));
+    sim->profiled_steps = 0;
+  }
+  return BPSX_OK;
+}
+
+int bpsx_get_kernel_times(bpsx_sim* sim, double* out_ms_sum, uint64_t* out_steps) {
+  if (!sim || !out_ms_sum || !out_steps) return fail(BPSX_E_INVAL, "get_kernel_times: null argument");
+  memcpy(out_ms_sum, sim->kernel_ms, sizeof(sim->kernel_ms));
+  *out_steps = sim->profiled_steps;
+  return BPSX_OK;
+}
+
+const char* bpsx_kernel_name(uint32_t idx) { return idx < BPSX_NUM_KERNELS ? kKernelNames[idx] : ""; }
+
+// ---- batched PathFinder-level queries: host arrays in, host arrays out
+static int batch_reserve(bpsx_sim* sim, size_t bytes) {
+  if (bytes <= sim->batch_bytes) return BPSX_OK;
+  if (sim->d_batch) HIP_TRY(hipFree(sim->d_batch));
+  sim->d_batch = nullptr;
+  sim->batch_bytes = 0;
+  HIP_TRY(hipMalloc(&sim->d_batch, bytes));
+  sim->batch_bytes = bytes;
+  return BPSX_OK;
+}
+static int check_scene(bpsx_sim* sim, uint32_t scene, const char* what) {
+  if (!sim || !sim->finalized) return fail(BPSX_E_STATE, std::string(what) + ": simulator not finalized");
+  if (scene >= sim->scenes.size()) return fail(BPSX_E_INVAL, std::string(what) + ": scene out of range");
+  for (auto& g : sim->groups)
+    if (g.in_flight) return fail(BPSX_E_STATE, std::string(what) + ": a step is in flight");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  return BPSX_OK;
+}
+
+int bpsx_snap_points(bpsx_sim* sim, uint32_t scene, const float* pts, uint32_t n, float* out_xyz, uint32_t* out_ref) {
+  int rc = check_scene(sim, scene, "snap_points");
+  if (rc) return rc;
+  if (!n) return BPSX_OK;
+  if (!pts || !out_xyz || !out_ref) return fail(BPSX_E_INVAL, "snap_points: null argument");
+  const size_t f3 = (size_t)n * 12;
+  if ((rc = batch_reserve(sim, 2 * f3 + (size_t)n * 4))) return rc;
+  char* b = (char*)sim->d_batch;
+  float* d_in = (float*)b; float* d_xyz = (float*)(b + f3); uint32_t* d_ref = (uint32_t*)(b + 2 * f3);
+  HIP_TRY(hipMemcpy(d_in, pts, f3, hipMemcpyHostToDevice));
+  launch_snap_batch(sim->nav, scene, d_in, n, d_xyz, d_ref, nullptr);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpy(out_xyz, d_xyz, f3, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(out_ref, d_ref, (size_t)n * 4, hipMemcpyDeviceToHost));
+  return BPSX_OK;
+}
+
+int bpsx_try_steps(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const uint32_t* start_ref, const float* end_xyz,
+                   uint32_t n, float* out_xyz, uint32_t* out_ref) {
+  int rc = check_scene(sim, scene, "try_steps");
+  if (rc) return rc;
+  if (!n) return BPSX_OK;
+  if (!start_xyz || !start_ref || !end_xyz || !out_xyz || !out_ref) return fail(BPSX_E_INVAL, "try_steps: null argument");
+  const size_t f3 = (size_t)n * 12, u1 = (size_t)n * 4;
+  if ((rc = batch_reserve(sim, 3 * f3 + 2 * u1))) return rc;
+  char* b = (char*)sim->d_batch;
+  float* d_s = (float*)b; float* d_e = (float*)(b + f3); float* d_o = (float*)(b + 2 * f3);
+  uint32_t* d_sr = (uint32_t*)(b + 3 * f3); uint32_t* d_or = (uint32_t*)(b + 3 * f3 + u1);
+  HIP_TRY(hipMemcpy(d_s, start_xyz, f3, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(d_e, end_xyz, f3, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(d_sr, start_ref, u1, hipMemcpyHostToDevice));
+  launch_try_step_batch(sim->nav, scene, d_s, d_sr, d_e, n, d_o, d_or, nullptr);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpy(out_xyz, d_o, f3, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(out_ref, d_or, u1, hipMemcpyDeviceToHost));
+  return BPSX_OK;
+}
+
+int bpsx_geodesic(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const uint32_t* start_ref, const float* end_xyz,
+                  const uint32_t* end_ref, uint32_t n, float* out_dist) {
+  int rc = check_scene(sim, scene, "geodesic");
+  if (rc) return rc;
+  if (!n) return BPSX_OK;
+  if (!start_xyz || !start_ref || !end_xyz || !end_ref || !out_dist) return fail(BPSX_E_INVAL, "geodesic: null argument");
+  const size_t f3 = (size_t)n * 12, u1 = (size_t)n * 4, qb = (size_t)n * sizeof(GeoQuery);
+  if ((rc = batch_reserve(sim, 2 * f3 + 3 * u1 + qb + 64))) return rc;
+  char* b = (char*)sim->d_batch;
+  GeoQuery* d_q = (GeoQuery*)b;  // first: keeps the 4-byte members aligned trivially
+  float* d_s = (float*)(b + qb); float* d_e = (float*)(b + qb + f3);
+  uint32_t* d_sr = (uint32_t*)(b + qb + 2 * f3); uint32_t* d_er = (uint32_t*)(b + qb + 2 * f3 + u1);
+  float* d_o = (float*)(b + qb + 2 * f3 + 2 * u1);
+  HIP_TRY(hipMemcpy(d_s, start_xyz, f3, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(d_e, end_xyz, f3, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(d_sr, start_ref, u1, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(d_er, end_ref, u1, hipMemcpyHostToDevice));
+  launch_geodesic_batch(sim->nav, scene, d_s, d_sr, d_e, d_er, n, d_q, sim->d_batch_counts, d_o, sim->d_slots,
+                        sim->geo_blocks, sim->d_counters, nullptr);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpy(out_dist, d_o, u1, hipMemcpyDeviceToHost));
+  return BPSX_OK;
+}
+
+int bpsx_random_points(bpsx_sim* sim, uint32_t scene, const float* u, uint32_t n, float* out_xyz, uint32_t* out_ref) {
+  int rc = check_scene(sim, scene, "random_points");
+  if (rc) return rc;
+  if (!n) return BPSX_OK;
+  if (!u || !out_xyz || !out_ref) return fail(BPSX_E_INVAL, "random_points: null argument");
+  const size_t f3 = (size_t)n * 12;
+  if ((rc = batch_reserve(sim, 2 * f3 + (size_t)n * 4))) return rc;
+  char* b = (char*)sim->d_batch;
+  float* d_in = (float*)b; float* d_xyz = (float*)(b + f3); uint32_t* d_ref = (uint32_t*)(b + 2 * f3);
+  HIP_TRY(hipMemcpy(d_in, u, f3, hipMemcpyHostToDevice));
+  launch_random_points(sim->nav, scene, d_in, n, d_xyz, d_ref, nullptr);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipMemcpy(out_xyz, d_xyz, f3, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(out_ref, d_ref, (size_t)n * 4, hipMemcpyDeviceToHost));
+  return BPSX_OK;
+}
+
+}  // extern "C"

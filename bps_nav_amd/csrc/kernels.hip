@@ -1,0 +1,434 @@
+// HIP kernels of the batch environment step (gfx950) and their launch wrappers.
+//
+// One step of a group of n agents is six launches on one stream:
+//   step_move      lane per agent: action, turn / forward move with wall sliding, polar
+//                  observation, and a geodesic query (goal -> agent) when the agent moved or
+//                  the episode ended                     (simulator.cpp:620-632, 651-710)
+//   geodesic       group of lanes per query: A* + funnel (PathFinder.cpp:485-541)
+//   step_finish    lane per agent: info, reward, mask; a finished episode picks its next
+//                  episode and is queued for reset      (simulator.cpp:634-641, 758-822, 601-610)
+//   reset_snap     lane per queued agent: snap start and goal, polar, query (agent -> goal)
+//                                                        (simulator.cpp:611-614, 744-751)
+//   geodesic       the reset queries
+//   reset_finish   lane per queued agent: initial distance bookkeeping (simulator.cpp:749-755, 801-806)
+#include <hip/hip_runtime.h>
+
+#include "geodesic_device.h"
+#include "kernels.h"
+
+namespace bpsx {
+
+namespace {
+
+// ---- counter-based reset stream (identical integer arithmetic on host and device)
+BPSX_DEV uint64_t mix64(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+BPSX_DEV uint64_t reset_key(uint64_t seed, uint32_t env, uint32_t count) {
+  return mix64(seed + 0x9E3779B97F4A7C15ull * ((uint64_t)env + 1) + 0xD1B54A32D192ED03ull * ((uint64_t)count + 1));
+}
+BPSX_DEV uint32_t reset_draw(uint64_t key, uint32_t k) {
+  return (uint32_t)(mix64(key + 0x9E3779B97F4A7C15ull * ((uint64_t)k + 1)) >> 32);
+}
+BPSX_DEV uint32_t draw_index(uint32_t r, uint32_t n) { return (uint32_t)(((uint64_t)r * (uint64_t)n) >> 32); }
+BPSX_DEV float draw_unit(uint32_t r) { return (float)(r >> 8) * (1.0f / 16777216.0f); }
+
+// ---- glm closed forms, quaternions stored x,y,z,w
+BPSX_DEV void quat_mul(const float* p, const float* q, float* o) {
+  const float w = p[3] * q[3] - p[0] * q[0] - p[1] * q[1] - p[2] * q[2];
+  const float x = p[3] * q[0] + p[0] * q[3] + p[1] * q[2] - p[2] * q[1];
+  const float y = p[3] * q[1] + p[1] * q[3] + p[2] * q[0] - p[0] * q[2];
+  const float z = p[3] * q[2] + p[2] * q[3] + p[0] * q[1] - p[1] * q[0];
+  o[0] = x; o[1] = y; o[2] = z; o[3] = w;
+}
+BPSX_DEV void cross3(const float* a, const float* b, float* o) {
+  o[0] = a[1] * b[2] - b[1] * a[2];
+  o[1] = a[2] * b[0] - b[2] * a[0];
+  o[2] = a[0] * b[1] - b[0] * a[1];
+}
+BPSX_DEV void quat_rotate(const float* q, const float* v, float* o) {
+  float uv[3], uuv[3];
+  cross3(q, v, uv);
+  cross3(q, uv, uuv);
+  for (int k = 0; k < 3; ++k) o[k] = v[k] + ((uv[k] * q[3]) + uuv[k]) * 2.0f;
+}
+// polar observation (rho, -phi) of the goal in the agent's frame (simulator.cpp:666-676)
+BPSX_DEV void write_polar(const AgentArrays& A, uint32_t gi, const float* pos, const float* q, const float* goal) {
+  const float v[3] = {goal[0] - pos[0], goal[1] - pos[1], goal[2] - pos[2]};
+  const float qxx = q[0] * q[0], qyy = q[1] * q[1], qzz = q[2] * q[2];
+  const float qxz = q[0] * q[2], qxy = q[0] * q[1], qyz = q[1] * q[2];
+  const float qwx = q[3] * q[0], qwy = q[3] * q[1], qwz = q[3] * q[2];
+  const float m00 = 1.0f - 2.0f * (qyy + qzz), m01 = 2.0f * (qxy + qwz), m02 = 2.0f * (qxz - qwy);
+  const float m20 = 2.0f * (qxz + qwy), m21 = 2.0f * (qyz - qwx), m22 = 1.0f - 2.0f * (qxx + qyy);
+  const float vx = m00 * v[0] + m01 * v[1] + m02 * v[2];
+  const float vz = m20 * v[0] + m21 * v[1] + m22 * v[2];
+  const float x = -vz, y = vx;
+  A.polars[(size_t)gi * 2 + 0] = sqrtf(x * x + y * y);
+  A.polars[(size_t)gi * 2 + 1] = -atan2f(y, x);
+}
+
+// Appends one item per lane with `pred` to a queue: one atomic per wavefront.
+BPSX_DEV uint32_t wave_append(bool pred, uint32_t* counter) {
+  const unsigned long long m = __ballot(pred);
+  if (!m) return 0;
+  const int lane = (int)(threadIdx.x & 63);
+  const int leader = __ffsll((long long)m) - 1;
+  uint32_t base = 0;
+  if (lane == leader) base = atomicAdd(counter, (uint32_t)__popcll(m));
+  base = (uint32_t)__shfl((int)base, leader);
+  return base + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
+}
+
+BPSX_DEV void load3(const float* p, size_t i, float* o) { o[0] = p[i * 3]; o[1] = p[i * 3 + 1]; o[2] = p[i * 3 + 2]; }
+BPSX_DEV void store3(float* p, size_t i, const float* v) { p[i * 3] = v[0]; p[i * 3 + 1] = v[1]; p[i * 3 + 2] = v[2]; }
+
+__global__ void k_clear_queues(StepQueues Q) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    Q.counts[0] = 0; Q.counts[1] = 0; Q.counts[2] = 0; Q.counts[3] = 0; Q.counts[4] = 0; Q.counts[5] = 0;
+  }
+}
+
+__global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, StepQueues Q, StepParams P,
+                                                   const int64_t* __restrict__ actions) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  bool want = false;
+  GeoQuery q{};
+  uint32_t movePolys = 0;
+  if (i < P.n) {
+    const uint32_t gi = P.base + i;
+    const int64_t action = actions[i];
+    if (action < 0 || action > 3) {
+      // the reference aborts here (simulator.cpp:704-708); flag it and leave the agent alone
+      atomicOr(P.error_flag, 1u);
+      A.flags[gi] = kAgentSkip;
+    } else {
+      const uint32_t step = A.step[gi] + 1;
+      A.step[gi] = step;
+      bool done = (float)step >= P.max_steps;
+      bool moved = false;
+      if (action == 0) {
+        done = true;
+      } else {
+        float pos[3], rot[4], goal[3];
+        load3(A.pos, gi, pos);
+        load3(A.goal, gi, goal);
+        for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
+        if (action == 1) {
+          const float fwd[3] = {0.f * 0.25f, 0.f * 0.25f, -1.f * 0.25f};
+          float delta[3];
+          quat_rotate(rot, fwd, delta);
+          const SceneDev& s = nav.scenes[A.scene[gi]];
+          NavPt st;
+          st.x = A.nav_xyz[(size_t)gi * 3]; st.y = A.nav_xyz[(size_t)gi * 3 + 1]; st.z = A.nav_xyz[(size_t)gi * 3 + 2];
+          st.ref = A.nav_ref[gi];
+          const NavPt r = try_step(nav, s, st, pos[0] + delta[0], pos[1] + delta[1], pos[2] + delta[2], &movePolys);
+          pos[0] = r.x; pos[1] = r.y; pos[2] = r.z;
+          store3(A.nav_xyz, gi, pos);
+          A.nav_ref[gi] = r.ref;
+          store3(A.pos, gi, pos);
+          moved = true;
+        } else {
+          quat_mul(rot, action == 2 ? P.turn_left : P.turn_right, rot);
+          for (int k = 0; k < 4; ++k) A.rot[(size_t)gi * 4 + k] = rot[k];
+        }
+        write_polar(A, gi, pos, rot, goal);
+      }
+      A.flags[gi] = (done ? kAgentDone : 0u) | (moved ? kAgentMoved : 0u);
+      if (done || moved) {
+        want = true;
+        load3(A.goal_xyz, gi, q.a);
+        q.a_ref = A.goal_ref[gi];
+        load3(A.nav_xyz, gi, q.b);
+        q.b_ref = A.nav_ref[gi];
+        q.scene = A.scene[gi];
+        q.out = gi;
+      }
+    }
+  }
+  const uint32_t slot = wave_append(want, &Q.counts[kQStepGeo]);
+  if (want) Q.step_queries[slot] = q;
+  // counters, one atomic per wavefront
+  const unsigned long long mv = __ballot(movePolys != 0);
+  uint32_t mp = movePolys;
+  for (int o = 32; o > 0; o >>= 1) mp += (uint32_t)__shfl_xor((int)mp, o);
+  if ((threadIdx.x & 63) == 0) {
+    if (mv) {
+      atomicAdd((unsigned long long*)&P.counters[kCntForward], (unsigned long long)__popcll(mv));
+      atomicAdd((unsigned long long*)&P.counters[kCntMovePolys], (unsigned long long)mp);
+    }
+  }
+  if (i == 0) atomicAdd((unsigned long long*)&P.counters[kCntSteps], (unsigned long long)P.n);
+}
+
+// Picks the next episode of agent gi and writes its pose; the snaps follow in reset_snap.
+BPSX_DEV void begin_reset(const NavData& nav, const AgentArrays& A, const StepParams& P, uint32_t gi) {
+  const uint32_t count = A.nresets[gi];
+  A.nresets[gi] = count + 1;
+  A.step[gi] = 1;
+  const uint32_t sc = A.scene[gi];
+  const SceneDev& s = nav.scenes[sc];
+  const uint64_t key = reset_key(P.seed, gi, count);
+  float ep[10];
+  if (P.reset_mode == 0) {
+    const uint32_t e = draw_index(reset_draw(key, 0), s.ep_count);
+    A.episode[gi] = e;
+    for (int k = 0; k < 10; ++k) ep[k] = nav.episodes[(size_t)(s.ep_base + e) * 10 + k];
+  } else {
+    A.episode[gi] = 0;
+    float a[3] = {0, 0, 0}, b[3] = {0, 0, 0};
+    uint32_t ip;
+    sample_point(nav, s, draw_unit(reset_draw(key, 0)), draw_unit(reset_draw(key, 1)), draw_unit(reset_draw(key, 2)), a, &ip);
+    sample_point(nav, s, draw_unit(reset_draw(key, 3)), draw_unit(reset_draw(key, 4)), draw_unit(reset_draw(key, 5)), b, &ip);
+    const uint32_t turns = draw_index(reset_draw(key, 6), 36);
+    float q[4] = {0, 0, 0, 1};
+    for (uint32_t t = 0; t < turns; ++t) quat_mul(q, P.turn_left, q);
+    ep[0] = a[0]; ep[1] = a[1]; ep[2] = a[2];
+    ep[3] = q[0]; ep[4] = q[1]; ep[5] = q[2]; ep[6] = q[3];
+    ep[7] = b[0]; ep[8] = b[1]; ep[9] = b[2];
+  }
+  store3(A.pos, gi, ep);
+  for (int k = 0; k < 4; ++k) A.rot[(size_t)gi * 4 + k] = ep[3 + k];
+  store3(A.goal, gi, ep + 7);
+}
+
+__global__ __launch_bounds__(256) void k_step_finish(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  bool reset = false;
+  uint32_t gi = 0;
+  if (i < P.n) {
+    gi = P.base + i;
+    const uint32_t f = A.flags[gi];
+    if (!(f & kAgentSkip)) {
+      const bool done = f & kAgentDone, moved = f & kAgentMoved;
+      float dist, success = 0, spl = 0;
+      if (done) {
+        dist = A.geo[gi];
+        success = dist < 0.2f ? 1.0f : 0.0f;
+        const float init = A.init[gi], cum = A.cum[gi];
+        const float mx = init < cum ? cum : init;
+        spl = success * init / mx;
+      } else if (moved) {
+        dist = A.geo[gi];
+        float pos[3], pp[3];
+        load3(A.pos, gi, pos);
+        load3(A.prev_pos, gi, pp);
+        const float dx = pos[0] - pp[0], dy = pos[1] - pp[1], dz = pos[2] - pp[2];
+        A.cum[gi] = A.cum[gi] + sqrtf(dx * dx + dy * dy + dz * dz);
+        A.info_prev[gi] = dist;
+        store3(A.prev_pos, gi, pos);
+      } else {
+        dist = A.info_prev[gi];
+      }
+      float reward = -1e-2f;
+      if (done) reward += 2.5f * spl;
+      else reward += A.rew_prev[gi] - dist;
+      A.rew_prev[gi] = dist;
+      A.rewards[gi] = reward;
+      A.masks[gi] = done ? 0 : 1;
+      A.infos[(size_t)gi * 3 + 0] = success;
+      A.infos[(size_t)gi * 3 + 1] = spl;
+      A.infos[(size_t)gi * 3 + 2] = dist;
+      if (done) {
+        begin_reset(nav, A, P, gi);
+        reset = true;
+      }
+    }
+  }
+  const uint32_t slot = wave_append(reset, &Q.counts[kQReset]);
+  if (reset) Q.reset_list[slot] = gi;
+}
+
+__global__ __launch_bounds__(256) void k_reset_all(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= P.n) return;
+  const uint32_t gi = P.base + i;
+  begin_reset(nav, A, P, gi);
+  Q.reset_list[i] = gi;
+  if (i == 0) Q.counts[kQReset] = P.n;
+}
+
+__global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t n = Q.counts[kQReset];
+  uint32_t cands = 0;
+  if (i < n) {
+    const uint32_t gi = Q.reset_list[i];
+    const SceneDev& s = nav.scenes[A.scene[gi]];
+    float pos[3], goal[3], rot[4];
+    load3(A.pos, gi, pos);
+    load3(A.goal, gi, goal);
+    for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
+    const NavPt a = snap_point(nav, s, pos[0], pos[1], pos[2], &cands);
+    const NavPt b = snap_point(nav, s, goal[0], goal[1], goal[2], &cands);
+    const float axyz[3] = {a.x, a.y, a.z}, bxyz[3] = {b.x, b.y, b.z};
+    store3(A.nav_xyz, gi, axyz);
+    A.nav_ref[gi] = a.ref;
+    store3(A.goal_xyz, gi, bxyz);
+    A.goal_ref[gi] = b.ref;
+    write_polar(A, gi, pos, rot, goal);
+    GeoQuery q;
+    q.a[0] = a.x; q.a[1] = a.y; q.a[2] = a.z; q.a_ref = a.ref;
+    q.b[0] = b.x; q.b[1] = b.y; q.b[2] = b.z; q.b_ref = b.ref;
+    q.scene = A.scene[gi];
+    q.out = gi;
+    Q.reset_queries[i] = q;
+    if (i == 0) {
+      Q.counts[kQResetGeo] = n;
+      atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
+    }
+    atomicAdd((unsigned long long*)&P.counters[kCntSnapCands], (unsigned long long)cands);
+  }
+}
+
+__global__ __launch_bounds__(256) void k_reset_finish(AgentArrays A, StepQueues Q) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= Q.counts[kQReset]) return;
+  const uint32_t gi = Q.reset_list[i];
+  const float d = A.geo[gi];
+  A.cum[gi] = 0;
+  A.init[gi] = d;
+  A.info_prev[gi] = d;
+  A.rew_prev[gi] = d;
+  float pos[3];
+  load3(A.pos, gi, pos);
+  store3(A.prev_pos, gi, pos);
+}
+
+template <int G>
+__global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries,
+                                                 const uint32_t* __restrict__ count, uint32_t* head, float* out,
+                                                 GeoSlot* slots, uint64_t* counters) {
+  constexpr int GPW = 64 / G;
+  __shared__ HeapEntry s_heap[GPW][kHeapLds];
+  __shared__ uint16_t s_first[GPW][kHashSize];
+  GeoGroup<G> g;
+  g.lane = (int)(threadIdx.x % G);
+  g.grp = (int)(threadIdx.x / G);
+  g.heap_lds = s_heap[g.grp];
+  g.first = s_first[g.grp];
+  g.ws = &slots[(size_t)blockIdx.x * GPW + g.grp];
+  g.heapSize = 0;
+  g.nodeCount = 0;
+  const uint32_t nq = *count;
+  uint32_t pops = 0, corridor = 0, done = 0;
+  for (;;) {
+    uint32_t qi = 0;
+    if (g.lane == 0) qi = atomicAdd(head, 1u);
+    qi = (uint32_t)__shfl((int)qi, 0, G);
+    if (qi >= nq) break;
+    const GeoQuery q = queries[qi];
+    const float d = geodesic_query<G>(g, nav, q, &pops, &corridor);
+    if (g.lane == 0) out[q.out] = d;
+    done++;
+  }
+  if (g.lane == 0 && done) {
+    atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)done);
+    atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)pops);
+    atomicAdd((unsigned long long*)&counters[kCntCorridor], (unsigned long long)corridor);
+  }
+}
+
+// ---- batched PathFinder-level kernels (one lane per item, or one group per item)
+__global__ void k_snap_batch(NavData nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  uint32_t c = 0;
+  const NavPt r = snap_point(nav, nav.scenes[scene], pts[(size_t)i * 3], pts[(size_t)i * 3 + 1], pts[(size_t)i * 3 + 2], &c);
+  oxyz[(size_t)i * 3] = r.x; oxyz[(size_t)i * 3 + 1] = r.y; oxyz[(size_t)i * 3 + 2] = r.z;
+  oref[i] = r.ref;
+}
+__global__ void k_try_step_batch(NavData nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
+                                 uint32_t n, float* oxyz, uint32_t* oref) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  uint32_t c = 0;
+  NavPt st{sxyz[(size_t)i * 3], sxyz[(size_t)i * 3 + 1], sxyz[(size_t)i * 3 + 2], sref[i]};
+  const NavPt r = try_step(nav, nav.scenes[scene], st, exyz[(size_t)i * 3], exyz[(size_t)i * 3 + 1], exyz[(size_t)i * 3 + 2], &c);
+  oxyz[(size_t)i * 3] = r.x; oxyz[(size_t)i * 3 + 1] = r.y; oxyz[(size_t)i * 3 + 2] = r.z;
+  oref[i] = r.ref;
+}
+__global__ void k_make_queries(uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
+                               const uint32_t* eref, uint32_t n, GeoQuery* q) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  GeoQuery o;
+  for (int k = 0; k < 3; ++k) { o.a[k] = sxyz[(size_t)i * 3 + k]; o.b[k] = exyz[(size_t)i * 3 + k]; }
+  o.a_ref = sref[i]; o.b_ref = eref[i]; o.scene = scene; o.out = i;
+  q[i] = o;
+}
+__global__ void k_random_points(NavData nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const SceneDev& s = nav.scenes[scene];
+  float p[3] = {0, 0, 0};
+  uint32_t ip = 0;
+  const bool ok = sample_point(nav, s, u[(size_t)i * 3], u[(size_t)i * 3 + 1], u[(size_t)i * 3 + 2], p, &ip);
+  oxyz[(size_t)i * 3] = p[0]; oxyz[(size_t)i * 3 + 1] = p[1]; oxyz[(size_t)i * 3 + 2] = p[2];
+  oref[i] = ok ? (s.ref_base | ip) : 0;
+}
+__global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
+
+}  // namespace
+
+// ------------------------------------------------------------------ launch wrappers
+static inline dim3 grid_for(uint32_t n, uint32_t block) { return dim3((n + block - 1) / block); }
+
+void launch_geodesic(const NavData& nav, const GeoQuery* queries, const uint32_t* count, uint32_t* head, float* out,
+                     GeoSlot* slots, uint32_t num_blocks, uint64_t* counters, hipStream_t st) {
+  // head is cleared by k_clear_queues / k_set_u32 before the producer kernel runs
+  hipLaunchKernelGGL(k_geodesic<kGeoGroup>, dim3(num_blocks), dim3(64), 0, st, nav, queries, count, head, out, slots, counters);
+}
+
+void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
+                 const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, hipStream_t st, hipEvent_t* ev) {
+  int e = 0;
+  auto mark = [&]() { if (ev) (void)hipEventRecord(ev[e++], st); };
+  mark();
+  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
+  hipLaunchKernelGGL(k_step_move, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P, actions_dev);
+  mark();
+  launch_geodesic(nav, Q.step_queries, &Q.counts[kQStepGeo], &Q.counts[kQStepGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  mark();
+  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
+  mark();
+  hipLaunchKernelGGL(k_reset_snap, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P);
+  mark();
+  launch_geodesic(nav, Q.reset_queries, &Q.counts[kQResetGeo], &Q.counts[kQResetGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  mark();
+  hipLaunchKernelGGL(k_reset_finish, grid_for(P.n, 256), dim3(256), 0, st, A, Q);
+  mark();
+}
+
+void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P, GeoSlot* slots,
+                  uint32_t geo_blocks, hipStream_t st) {
+  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
+  hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
+  hipLaunchKernelGGL(k_reset_snap, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P);
+  launch_geodesic(nav, Q.reset_queries, &Q.counts[kQResetGeo], &Q.counts[kQResetGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  hipLaunchKernelGGL(k_reset_finish, grid_for(P.n, 256), dim3(256), 0, st, A, Q);
+}
+
+void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref,
+                       hipStream_t st) {
+  hipLaunchKernelGGL(k_snap_batch, grid_for(n, 64), dim3(64), 0, st, nav, scene, pts, n, oxyz, oref);
+}
+void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
+                           uint32_t n, float* oxyz, uint32_t* oref, hipStream_t st) {
+  hipLaunchKernelGGL(k_try_step_batch, grid_for(n, 64), dim3(64), 0, st, nav, scene, sxyz, sref, exyz, n, oxyz, oref);
+}
+void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
+                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [2] */, float* out,
+                           GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st) {
+  hipLaunchKernelGGL(k_make_queries, grid_for(n, 256), dim3(256), 0, st, scene, sxyz, sref, exyz, eref, n, qbuf);
+  hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, st, &count_head[0], n);
+  hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, st, &count_head[1], 0u);
+  launch_geodesic(nav, qbuf, &count_head[0], &count_head[1], out, slots, geo_blocks, counters, st);
+}
+void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,
+                          hipStream_t st) {
+  hipLaunchKernelGGL(k_random_points, grid_for(n, 64), dim3(64), 0, st, nav, scene, u, n, oxyz, oref);
+}
+
+}  // namespace bpsx

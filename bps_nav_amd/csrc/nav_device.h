@@ -1,0 +1,343 @@
+// Device-side navmesh queries on PolyRec records: the geometry primitives and the
+// per-lane queries (nearest polygon, move along surface, height) of the step path.
+// Compile with -ffp-contract=off: polygon ids must equal the reference's bit for bit, so
+// every expression keeps Detour's fp32 operation order and is never fused.
+//
+// Reference semantics followed (read, not copied):
+//   DetourCommon.cpp:170-184 (point-segment distance), :204-233 (height on triangle),
+//   :238-270 (point in polygon, edge distances), :332-369 (random point in polygon);
+//   DetourNavMesh.cpp:619-758 (height mesh queries); DetourNavMeshQuery.cpp:538-586
+//   (boundary clamp), :642-826 (nearest polygon over the BV tree), :2016-2255 (move along
+//   surface); PathFinder.cpp:24-44, 543-584 (snapPoint / tryStep conventions).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "device_types.h"
+
+namespace bpsx {
+
+#define BPSX_DEV __device__ __forceinline__
+
+struct NavPt {
+  float x, y, z;
+  uint32_t ref;
+};
+
+BPSX_DEV bool finite3(float x, float y, float z) { return isfinite(x) && isfinite(y) && isfinite(z); }
+
+BPSX_DEV float dist_pt_seg_sqr2d(float px, float pz, const float* p, const float* q, float& t) {
+  const float pqx = q[0] - p[0], pqz = q[2] - p[2];
+  float dx = px - p[0], dz = pz - p[2];
+  const float d = pqx * pqx + pqz * pqz;
+  t = pqx * dx + pqz * dz;
+  if (d > 0) t /= d;
+  if (t < 0) t = 0;
+  else if (t > 1) t = 1;
+  dx = p[0] + t * pqx - px;
+  dz = p[2] + t * pqz - pz;
+  return dx * dx + dz * dz;
+}
+
+BPSX_DEV bool point_in_poly(float px, float pz, const PolyRec& r) {
+  bool c = false;
+  const int nv = r.nv;
+  for (int i = 0, j = nv - 1; i < nv; j = i++) {
+    const float* vi = r.v[i];
+    const float* vj = r.v[j];
+    if (((vi[2] > pz) != (vj[2] > pz)) && (px < (vj[0] - vi[0]) * (pz - vi[2]) / (vj[2] - vi[2]) + vi[0])) c = !c;
+  }
+  return c;
+}
+
+BPSX_DEV bool height_on_triangle(float px, float pz, const float* a, const float* b, const float* c, float& h) {
+  const float EPS = 1e-6f;
+  const float v0x = c[0] - a[0], v0y = c[1] - a[1], v0z = c[2] - a[2];
+  const float v1x = b[0] - a[0], v1y = b[1] - a[1], v1z = b[2] - a[2];
+  const float v2x = px - a[0], v2z = pz - a[2];
+  float denom = v0x * v1z - v0z * v1x;
+  if (fabsf(denom) < EPS) return false;
+  float u = v1z * v2x - v1x * v2z;
+  float v = v0x * v2z - v0z * v2x;
+  if (denom < 0) { denom = -denom; u = -u; v = -v; }
+  if (u >= 0.0f && v >= 0.0f && (u + v) <= denom) {
+    h = a[1] + (v0y * u + v1y * v) / denom;
+    return true;
+  }
+  return false;
+}
+
+BPSX_DEV const float* detail_vert(const NavData& nav, const PolyRec& r, int k) {
+  return k < r.nv ? r.v[k] : &nav.dverts[(size_t)(r.dvert_base + (uint32_t)(k - r.nv)) * 3];
+}
+
+template <bool kOnlyBoundary>
+BPSX_DEV void closest_on_detail_edges(const NavData& nav, const PolyRec& r, float px, float py, float pz, float* out) {
+  float dmin = 3.402823466e+38f, tmin = 0;
+  const float* pmin = nullptr;
+  const float* pmax = nullptr;
+  for (int i = 0; i < r.tri_count; ++i) {
+    const uint8_t* tris = &nav.dtris[(size_t)(r.tri_base + i) * 4];
+    const uint8_t tf = tris[3];
+    if (kOnlyBoundary && (tf & 0x15) == 0) continue;
+    const float* v[3] = {detail_vert(nav, r, tris[0]), detail_vert(nav, r, tris[1]), detail_vert(nav, r, tris[2])};
+    for (int k = 0, j = 2; k < 3; j = k++) {
+      if ((((tf >> (j * 2)) & 1) == 0) && (kOnlyBoundary || tris[j] < tris[k])) continue;
+      float t;
+      const float d = dist_pt_seg_sqr2d(px, pz, v[j], v[k], t);
+      if (d < dmin) { dmin = d; tmin = t; pmin = v[j]; pmax = v[k]; }
+    }
+  }
+  if (!pmin) { out[0] = px; out[1] = py; out[2] = pz; return; }
+  out[0] = pmin[0] + (pmax[0] - pmin[0]) * tmin;
+  out[1] = pmin[1] + (pmax[1] - pmin[1]) * tmin;
+  out[2] = pmin[2] + (pmax[2] - pmin[2]) * tmin;
+}
+
+// dtNavMesh::getPolyHeight: false when (px,pz) is outside the polygon.
+BPSX_DEV bool poly_height(const NavData& nav, const PolyRec& r, float px, float py, float pz, float& h) {
+  if (r.type != 0) return false;
+  if (!point_in_poly(px, pz, r)) return false;
+  for (int j = 0; j < r.tri_count; ++j) {
+    const uint8_t* t = &nav.dtris[(size_t)(r.tri_base + j) * 4];
+    if (height_on_triangle(px, pz, detail_vert(nav, r, t[0]), detail_vert(nav, r, t[1]), detail_vert(nav, r, t[2]), h))
+      return true;
+  }
+  float c[3];
+  closest_on_detail_edges<false>(nav, r, px, py, pz, c);
+  h = c[1];
+  return true;
+}
+
+// closestPointOnPolyBoundary: the point itself when inside (xz), else its projection onto
+// the nearest polygon edge.
+BPSX_DEV void closest_on_poly_boundary(const PolyRec& r, const float* pos, float* out) {
+  float ed[kNvp], et[kNvp];
+  bool c = false;
+  const int nv = r.nv;
+  for (int i = 0, j = nv - 1; i < nv; j = i++) {
+    const float* vi = r.v[i];
+    const float* vj = r.v[j];
+    if (((vi[2] > pos[2]) != (vj[2] > pos[2])) &&
+        (pos[0] < (vj[0] - vi[0]) * (pos[2] - vi[2]) / (vj[2] - vi[2]) + vi[0]))
+      c = !c;
+    ed[j] = dist_pt_seg_sqr2d(pos[0], pos[2], vj, vi, et[j]);
+  }
+  if (c) { out[0] = pos[0]; out[1] = pos[1]; out[2] = pos[2]; return; }
+  float dmin = ed[0];
+  int imin = 0;
+  for (int i = 1; i < nv; ++i)
+    if (ed[i] < dmin) { dmin = ed[i]; imin = i; }
+  const float* va = r.v[imin];
+  const float* vb = r.v[(imin + 1) % nv];
+  const float t = et[imin];
+  out[0] = va[0] + (vb[0] - va[0]) * t;
+  out[1] = va[1] + (vb[1] - va[1]) * t;
+  out[2] = va[2] + (vb[2] - va[2]) * t;
+}
+
+// Polygon index of a ref within its scene, or kInvalidPoly (dtNavMesh::isValidPolyRef).
+BPSX_DEV uint32_t decode_ref(const SceneDev& s, uint32_t ref) {
+  if (!ref) return kInvalidPoly;
+  const uint32_t ip = ref & s.poly_mask;
+  if ((ref & ~s.poly_mask) != s.ref_base || ip >= s.poly_count) return kInvalidPoly;
+  return ip;
+}
+
+// One candidate of the nearest-polygon search: distance rule of dtFindNearestPolyQuery.
+BPSX_DEV float snap_candidate(const NavData& nav, const SceneDev& s, const PolyRec& r, float px, float py, float pz,
+                              float* cp) {
+  float h;
+  if (poly_height(nav, r, px, py, pz, h)) {
+    cp[0] = px; cp[1] = h; cp[2] = pz;
+    float d = fabsf(py - h) - s.climb;
+    return d > 0 ? d * d : 0;
+  }
+  closest_on_detail_edges<true>(nav, r, px, py, pz, cp);
+  const float dx = px - cp[0], dy = py - cp[1], dz = pz - cp[2];
+  return dx * dx + dy * dy + dz * dz;
+}
+
+struct SnapBox {
+  uint16_t bmin[3], bmax[3];
+  bool hit_tile;
+};
+BPSX_DEV float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+BPSX_DEV SnapBox snap_box(const SceneDev& s, float px, float py, float pz) {
+  SnapBox b;
+  const float qmin[3] = {px - 2.0f, py - 4.0f, pz - 2.0f};
+  const float qmax[3] = {px + 2.0f, py + 4.0f, pz + 2.0f};
+  const int minx = (int)floorf((qmin[0] - s.orig[0]) / s.tile_w), miny = (int)floorf((qmin[2] - s.orig[2]) / s.tile_h);
+  const int maxx = (int)floorf((qmax[0] - s.orig[0]) / s.tile_w), maxy = (int)floorf((qmax[2] - s.orig[2]) / s.tile_h);
+  b.hit_tile = !(s.tx < minx || s.tx > maxx || s.ty < miny || s.ty > maxy);
+  for (int k = 0; k < 3; ++k) {
+    const float lo = clampf(qmin[k], s.bmin[k], s.bmax[k]) - s.bmin[k];
+    const float hi = clampf(qmax[k], s.bmin[k], s.bmax[k]) - s.bmin[k];
+    b.bmin[k] = (uint16_t)((uint16_t)(int)(s.qfac * lo) & 0xfffe);
+    b.bmax[k] = (uint16_t)((uint16_t)(int)(s.qfac * hi + 1) | 1);
+  }
+  return b;
+}
+
+// snapPoint, one lane per point: BV-tree walk with escape indices, candidates taken in tree
+// order with a strict '<' so the first of equally near polygons wins.
+BPSX_DEV NavPt snap_point(const NavData& nav, const SceneDev& s, float px, float py, float pz, uint32_t* ncand) {
+  const float qnan = __int_as_float(0x7fc00000);
+  NavPt out{qnan, qnan, qnan, 0};
+  if (!finite3(px, py, pz)) return out;
+  const SnapBox box = snap_box(s, px, py, pz);
+  if (!box.hit_tile) return out;
+  float best = 3.402823466e+38f;
+  float bp[3] = {0, 0, 0};
+  uint32_t bestIp = kInvalidPoly;
+  uint32_t i = 0;
+  while (i < s.bv_count) {
+    const BVNodeDev nd = nav.bv[s.bv_base + i];
+    bool overlap = true;
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+      if (box.bmin[k] > nd.bmax[k] || box.bmax[k] < nd.bmin[k]) overlap = false;
+    const bool leaf = nd.i >= 0;
+    if (leaf && overlap) {
+      const PolyRec& r = nav.polys[s.poly_base + (uint32_t)nd.i];
+      if (r.flags & 1) {
+        float cp[3];
+        const float d = snap_candidate(nav, s, r, px, py, pz, cp);
+        (*ncand)++;
+        if (d < best) { best = d; bestIp = (uint32_t)nd.i; bp[0] = cp[0]; bp[1] = cp[1]; bp[2] = cp[2]; }
+      }
+    }
+    if (overlap || leaf) i++;
+    else i += (uint32_t)(-nd.i);
+  }
+  if (bestIp == kInvalidPoly || isnan(bp[0])) return out;
+  out.x = bp[0]; out.y = bp[1]; out.z = bp[2];
+  out.ref = s.ref_base | bestIp;
+  return out;
+}
+
+// tryStep with sliding, one lane per agent.
+BPSX_DEV NavPt try_step(const NavData& nav, const SceneDev& s, const NavPt& start, float ex, float ey, float ez,
+                        uint32_t* npolys) {
+  const uint32_t startIp = decode_ref(s, start.ref);
+  if (startIp == kInvalidPoly || !finite3(start.x, start.y, start.z) || !finite3(ex, ey, ez)) return start;
+  uint16_t nodeId[kTinyNodes];
+  uint64_t closed = 1ull;
+  int nnodes = 1;
+  uint8_t queue[kMoveQueue];
+  int nqueue = 1;
+  nodeId[0] = (uint16_t)startIp;
+  queue[0] = 0;
+  float bx = start.x, by = start.y, bz = start.z;
+  float bestDist = 3.402823466e+38f;
+  int bestNode = -1;
+  const float sx = start.x + (ex - start.x) * 0.5f, sz = start.z + (ez - start.z) * 0.5f;
+  const float ddx = ex - start.x, ddy = ey - start.y, ddz = ez - start.z;
+  const float sr = sqrtf(ddx * ddx + ddy * ddy + ddz * ddz) / 2.0f + 0.001f;
+  const float searchRadSqr = sr * sr;
+  while (nqueue) {
+    const int cur = queue[0];
+    for (int i = 0; i < nqueue - 1; ++i) queue[i] = queue[i + 1];
+    nqueue--;
+    const PolyRec& r = nav.polys[s.poly_base + nodeId[cur]];
+    (*npolys)++;
+    if (point_in_poly(ex, ez, r)) {
+      bestNode = cur;
+      bx = ex; by = ey; bz = ez;
+      break;
+    }
+    const int nv = r.nv;
+    for (int i = 0, j = nv - 1; i < nv; j = i++) {
+      // single-tile meshes carry no tile-border links, so a border edge is a wall
+      const uint16_t nb = (r.nei[j] & 0x8000) ? (uint16_t)0 : r.walk[j];
+      const float* vj = r.v[j];
+      const float* vi = r.v[i];
+      if (!nb) {
+        float t;
+        const float d = dist_pt_seg_sqr2d(ex, ez, vj, vi, t);
+        if (d < bestDist) {
+          bx = vj[0] + (vi[0] - vj[0]) * t;
+          by = vj[1] + (vi[1] - vj[1]) * t;
+          bz = vj[2] + (vi[2] - vj[2]) * t;
+          bestDist = d;
+          bestNode = cur;
+        }
+      } else {
+        const uint16_t ip = (uint16_t)(nb - 1);
+        int nn = -1;
+        for (int k = 0; k < nnodes; ++k)
+          if (nodeId[k] == ip) { nn = k; break; }
+        if (nn < 0) {
+          if (nnodes >= kTinyNodes) continue;
+          nn = nnodes++;
+          nodeId[nn] = ip;
+        }
+        if ((closed >> nn) & 1ull) continue;
+        float t;
+        const float d = dist_pt_seg_sqr2d(sx, sz, vj, vi, t);
+        if (d > searchRadSqr) continue;
+        if (nqueue < kMoveQueue) {
+          closed |= 1ull << nn;
+          queue[nqueue++] = (uint8_t)nn;
+        }
+      }
+    }
+  }
+  if (bestNode < 0) return start;
+  NavPt out{bx, by, bz, s.ref_base | (uint32_t)nodeId[bestNode]};
+  if (isfinite(bx) && isfinite(bz)) {
+    float h;
+    if (poly_height(nav, nav.polys[s.poly_base + nodeId[bestNode]], bx, by, bz, h)) out.y = h;
+  }
+  return out;
+}
+
+// dtRandomPointInConvexPoly on a polygon record.
+BPSX_DEV void random_point_in_poly(const PolyRec& r, float sv, float tv, float* out) {
+  float areas[kNvp];
+  float areasum = 0.0f;
+  const int n = r.nv;
+  for (int i = 2; i < n; i++) {
+    const float abx = r.v[i - 1][0] - r.v[0][0], abz = r.v[i - 1][2] - r.v[0][2];
+    const float acx = r.v[i][0] - r.v[0][0], acz = r.v[i][2] - r.v[0][2];
+    areas[i] = acx * abz - abx * acz;
+    areasum += areas[i] > 0.001f ? areas[i] : 0.001f;
+  }
+  const float thr = sv * areasum;
+  float acc = 0.0f, u = 1.0f;
+  int tri = n - 1;
+  for (int i = 2; i < n; i++) {
+    const float dacc = areas[i];
+    if (thr >= acc && thr < (acc + dacc)) { u = (thr - acc) / dacc; tri = i; break; }
+    acc += dacc;
+  }
+  const float v = sqrtf(tv);
+  const float a = 1 - v, b = (1 - u) * v, c = u * v;
+  const float* pa = r.v[0];
+  const float* pb = r.v[tri - 1];
+  const float* pc = r.v[tri];
+  out[0] = a * pa[0] + b * pb[0] + c * pc[0];
+  out[1] = a * pa[1] + b * pb[1] + c * pc[1];
+  out[2] = a * pa[2] + b * pb[2] + c * pc[2];
+}
+
+// Area-weighted polygon pick + point: first polygon whose inclusive area prefix sum exceeds
+// u0 * total, then a point inside it, y from the height mesh.
+BPSX_DEV bool sample_point(const NavData& nav, const SceneDev& s, float u0, float sv, float tv, float* out,
+                           uint32_t* out_ip) {
+  if (!(s.area_total > 0.0f)) return false;
+  const float target = u0 * s.area_total;
+  uint32_t lo = 0, hi = s.poly_count - 1;
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi) / 2;
+    if (nav.polys[s.poly_base + mid].area_cum > target) hi = mid;
+    else lo = mid + 1;
+  }
+  const PolyRec& r = nav.polys[s.poly_base + lo];
+  random_point_in_poly(r, sv, tv, out);
+  float h;
+  if (isfinite(out[0]) && isfinite(out[2]) && poly_height(nav, r, out[0], out[1], out[2], h)) out[1] = h;
+  *out_ip = lo;
+  return true;
+}
+
+}  // namespace bpsx

@@ -113,6 +113,8 @@ def config_scene(config, scene_idx):
                          door_width=0.9, wall=0.2, clutter_frac=0.15, box_min=0.5, box_max=1.5, tri_frac=0.1,
                          hex_frac=0.1)
     if config == 4:
-        return gen_scene(MAZE, seed, cell=5, maze_w=26, maze_h=26, corridor_min=1.0, corridor_max=1.5, wall=0.75,
+        # 0.5 m cells keep A* inside Detour's 2048-node pool and 256-polygon corridor limit for
+        # the 15-40 m episodes of this configuration (finer cells make the reference return inf)
+        return gen_scene(MAZE, seed, cell=10, maze_w=50, maze_h=50, corridor_min=1.0, corridor_max=1.5, wall=1.0,
                          braid=0.08, tri_frac=0.05, hex_frac=0.05)
     raise ValueError("config must be 1..4")

@@ -117,11 +117,14 @@ int bpsx_check_errors(bpsx_sim *sim);
  * [4] corridor polygons string-pulled, [5] resets, [6] polygons visited by moves. */
 #define BPSX_NUM_COUNTERS 8
 int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
-/* Name and average duration of the kernels timed with HIP events during the last
- * bpsx_profile_steps() call. */
-int bpsx_profile_steps(bpsx_sim *sim, uint32_t group, const int64_t *actions_dev,
-                       uint32_t num_steps, float *out_ms_per_kernel /* [BPSX_NUM_KERNELS] */);
+/* Per-kernel timing with HIP events on the step's own stream. While enabled, every
+ * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
+ * elapsed times up.  get_kernel_times returns the sums in milliseconds and the number of
+ * steps they cover; enabling clears the sums. */
 #define BPSX_NUM_KERNELS 6
+int bpsx_set_profiling(bpsx_sim *sim, int enabled);
+int bpsx_get_kernel_times(bpsx_sim *sim, double *out_ms_sum /* [BPSX_NUM_KERNELS] */,
+                          uint64_t *out_steps);
 const char *bpsx_kernel_name(uint32_t idx);
 
 /* ---- batched PathFinder queries on one uploaded scene (PathFinder.h:99-227) ----

@@ -1,0 +1,25 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    from oracle import bpo
+    return bpo.load_oracle()
+
+
+@pytest.fixture(scope="session")
+def reflib():
+    """The compiled reference (oracle/_ref); None outside the development container."""
+    from oracle import bpo
+    return bpo.load_ref()

@@ -1,0 +1,135 @@
+"""GPU parity: the HIP engine, called through the C ABI, against the CPU oracle on the same
+seeded scenes, episodes and action streams.
+
+Bars (BASELINE.json): polygon ids, dones and resets bit-exact; positions within 1e-4 m,
+headings within 1e-4 rad; geodesic distance and reward within 1e-3 relative.  The kernels
+keep the reference's fp32 operation order, so everything except the polar angle (device
+atan2f vs glibc atan2f) is in fact compared bit for bit here.
+"""
+import numpy as np
+import pytest
+
+from tests import common
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch
+
+
+def make_gen(sc, n, **kw):
+    from bps_nav_amd.bps_sim import PointNavRolloutGenerator
+    return PointNavRolloutGenerator("", "", n, len(sc), scenes=sc, **kw)
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4])
+def test_batched_queries_match_oracle(oracle, torch_cuda, config):
+    from bps_nav_amd import scenes
+    from oracle import bpo
+    print(f"case: batched queries config {config}", flush=True)
+    blob = scenes.config_scene(config, 0)
+    nav = bpo.Nav(oracle, blob)
+    gen = make_gen([(blob, np.zeros((1, 10), np.float32))], 1)
+    rng = np.random.default_rng(config)
+    pts = scenes.sample_points(blob, 7, 3000)
+    q = pts + rng.normal(0, 0.3, pts.shape).astype(np.float32)
+    q[:, 1] += rng.uniform(-1, 2, len(q)).astype(np.float32)
+    q[:5] += 100.0  # far outside the mesh: snap fails
+    xo, ro = nav.snap(q)
+    xg, rg = gen.snap_points(0, q)
+    assert np.array_equal(ro, rg)
+    assert np.array_equal(common.bits(xo), common.bits(xg))
+    assert (ro[:5] == 0).all() and np.isnan(xg[:5]).all()
+    ok = ro != 0
+    ang = rng.uniform(0, 2 * np.pi, len(q))
+    d = rng.uniform(0, 0.6, len(q))
+    end = xo.copy()
+    end[:, 0] += (d * np.cos(ang)).astype(np.float32)
+    end[:, 2] += (d * np.sin(ang)).astype(np.float32)
+    so, sro = nav.try_step(xo[ok], ro[ok], end[ok])
+    sg, srg = gen.try_steps(0, xo[ok], ro[ok], end[ok])
+    assert np.array_equal(sro, srg)
+    assert np.array_equal(common.bits(so), common.bits(sg))
+    m = min(1000, ok.sum() // 2)
+    a, ar, b, br = xo[ok][:m], ro[ok][:m], xo[ok][m:2 * m], ro[ok][m:2 * m]
+    go = nav.geodesic(a, ar, b, br)
+    gg = gen.geodesic(0, a, ar, b, br)
+    assert np.array_equal(common.bits(go), common.bits(gg)), \
+        f"{(common.bits(go) != common.bits(gg)).sum()} of {m} geodesics differ"
+    # invalid refs and coincident points
+    gz = gen.geodesic(0, a[:4], ar[:4], a[:4], ar[:4])
+    assert (gz == 0).all()
+    gi = gen.geodesic(0, a[:4], np.zeros(4, np.uint32), b[:4], br[:4])
+    assert np.isinf(gi).all()
+    gen.close()
+
+
+@pytest.mark.parametrize("config,num_scenes,n,steps,mode", [
+    (1, 1, 64, 500, 0), (2, 4, 256, 300, 0), (3, 2, 128, 200, 1), (4, 4, 256, 200, 0), (2, 4, 256, 150, 1)])
+def test_step_parity(oracle, torch_cuda, config, num_scenes, n, steps, mode):
+    from oracle import bpo
+    print(f"case: step parity config {config} scenes {num_scenes} agents {n} mode {mode}", flush=True)
+    sc = common.build_scenes(oracle, config, num_scenes)
+    cpu = bpo.Sim(oracle, sc, n, reset_mode=mode, seed=11, threads=4)
+    gen = make_gen(sc, n, reset_mode=mode, seed=11)
+    cpu.reset()
+    gen.reset(0)
+    views = dict(rewards=gen.get_rewards(0), masks=gen.get_masks(0), polars=gen.get_polars(0))
+    infos = gen.get_infos(0)
+    state = gen.get_state(0)
+    acts = common.action_stream(config, steps, n)
+    dones = 0
+    for t, a in enumerate(acts):
+        cpu.step(a)
+        gen.step(0, torch_cuda.from_numpy(a).cuda() if t % 2 else a)  # device and host action paths
+        co, cs = cpu.outputs(), cpu.state()
+        g_state = {k: v.cpu().numpy() for k, v in state.items()}
+        for k in ("poly_ref", "goal_ref", "step", "episode", "num_resets"):
+            assert np.array_equal(cs[k], g_state[k].view(np.uint32)), f"{k} differs at step {t}"
+        assert np.array_equal(co["masks"], views["masks"].cpu().numpy()), f"dones differ at step {t}"
+        np.testing.assert_allclose(g_state["position"], cs["position"], atol=1e-4, rtol=0)
+        np.testing.assert_allclose(g_state["rotation"], cs["rotation"], atol=1e-6, rtol=0)
+        assert np.array_equal(common.bits(g_state["position"]), common.bits(cs["position"])), f"position bits at step {t}"
+        gi = infos.packed.cpu().numpy()
+        gr = views["rewards"].cpu().numpy()
+        np.testing.assert_allclose(gi, co["infos"], rtol=1e-3, atol=0, equal_nan=True)
+        np.testing.assert_allclose(gr, co["rewards"], rtol=1e-3, atol=1e-6, equal_nan=True)
+        assert np.array_equal(common.bits(gi), common.bits(co["infos"])) or np.isnan(gi).any(), f"info bits at step {t}"
+        gp = views["polars"].cpu().numpy()
+        np.testing.assert_allclose(gp[:, 0], co["polars"][:, 0], rtol=1e-6, atol=1e-6)
+        dphi = np.abs(gp[:, 1] - co["polars"][:, 1])
+        dphi = np.minimum(dphi, 2 * np.pi - dphi)
+        assert (dphi < 1e-4).all(), f"polar angle differs by {dphi.max()} rad at step {t}"
+        dones += int((co["masks"] == 0).sum())
+    assert dones > 0, "the stream never finished an episode: resets were not exercised"
+    gen.check_errors()
+    gen.close()
+
+
+def test_error_paths(oracle, torch_cuda):
+    print("case: error paths", flush=True)
+    sc = common.build_scenes(oracle, 1, 1, episodes_per_scene=8)
+    gen = make_gen(sc, 8)
+    gen.reset(0)
+    with pytest.raises(RuntimeError, match="no step in flight"):
+        gen.step_end(0)
+    a = np.ones(8, np.int64)
+    gen.step_start(0, a)
+    with pytest.raises(RuntimeError, match="previous step not finished"):
+        gen.step_start(0, a)
+    gen.step_end(0)
+    before = {k: v.clone() for k, v in gen.get_state(0).items()}
+    bad = np.array([1, 7, -1, 2, 1, 1, 1, 1], np.int64)
+    gen.step(0, bad)
+    after = gen.get_state(0)
+    for k in before:  # agents with invalid actions are left untouched
+        assert torch_cuda.equal(before[k][1:3], after[k][1:3])
+    with pytest.raises(RuntimeError, match="outside 0..3"):
+        gen.check_errors()
+    with pytest.raises(RuntimeError):
+        gen.rgba(0)
+    gen.close()
