@@ -153,7 +153,14 @@ class Sim {
     masks_.assign(numEnvs_, 0);
     infos_.assign((size_t)numEnvs_ * 3, 0.f);
     polars_.assign((size_t)numEnvs_ * 2, 0.f);
-    for (int t = 0; t < numThreads_; ++t) ctxs_.push_back(B::make_ctx(scenes_));
+    // every participant builds its own query contexts, concurrently, like the reference's
+    // worker threads do at start-up (simulator.cpp:1712-1738)
+    ctxs_.resize((size_t)numThreads_);
+    {
+      std::vector<std::thread> builders;
+      for (int t = 0; t < numThreads_; ++t) builders.emplace_back([this, t] { ctxs_[t] = B::make_ctx(scenes_); });
+      for (auto& b : builders) b.join();
+    }
     startWorkers();
     return true;
   }
