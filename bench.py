@@ -140,7 +140,7 @@ def main():
     # roofline of the dominant kernel (geodesic over the step's queries), HIP-event timed
     dominant = max(kt, key=kt.get)
     geo_bytes = BYTES_PER_CORRIDOR_POLY * d["corridor_polys"] + BYTES_PER_QUERY_ENDS * d["geodesic_queries"]
-    geo_ms = kt["geodesic_step"] + kt["geodesic_reset"]
+    geo_ms = kt["geodesic"]
     achieved = geo_bytes / K / (geo_ms * 1e-3) / 1e9 if geo_ms > 0 else 0.0
     roofline = {"bound": "hbm", "kernel": "k_geodesic", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS, "traffic": None, "dominant_kernel_by_time": dominant,

@@ -213,11 +213,11 @@ class PointNavRolloutGenerator:
 
     def kernel_times(self):
         """{kernel name: average ms per step} over the steps profiled so far, and the step count."""
-        ms = (C.c_double * 6)()
+        ms = (C.c_double * 4)()
         steps = C.c_uint64()
         _lib.check(self._L.bpsx_get_kernel_times(self._h, ms, C.byref(steps)))
         k = max(1, steps.value)
-        return {self._L.bpsx_kernel_name(i).decode(): ms[i] / k for i in range(6)}, steps.value
+        return {self._L.bpsx_kernel_name(i).decode(): ms[i] / k for i in range(4)}, steps.value
 
     # ---- batched PathFinder-level queries (host arrays)
     def snap_points(self, scene, pts):

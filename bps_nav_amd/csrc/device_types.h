@@ -37,11 +37,16 @@ struct alignas(128) PolyRec {
 };
 static_assert(sizeof(PolyRec) == 128, "PolyRec must be one cache line");
 
-struct BVNodeDev {  // dtBVNode
+// dtBVNode repacked at upload: same quantised bounds; a leaf carries its polygon index, an
+// internal node carries Detour's escape offset (for the in-order walk) and the index of its
+// right child (its left child is the next node), so a wavefront can descend level by level.
+struct BVNodeDev {
   uint16_t bmin[3], bmax[3];
-  int32_t i;
+  uint16_t a;   // leaf: polygon index; internal: escape offset
+  uint16_t b;   // leaf: 0xffff; internal: index of the right child
 };
 static_assert(sizeof(BVNodeDev) == 16, "BV node");
+constexpr uint16_t kBVLeaf = 0xffff;
 
 struct SceneDev {
   uint32_t poly_base, poly_count;
@@ -55,7 +60,8 @@ struct SceneDev {
   float qfac;                       // bvQuantFactor
   float climb;                      // walkableClimb
   float area_total;
-  uint32_t pad[3];
+  uint32_t bv_tree_ok;              // 1: child links verified, level-by-level descent allowed
+  uint32_t pad[2];
 };
 
 // ---- per-agent state, structure of arrays over all agents of the simulator
@@ -77,14 +83,14 @@ struct AgentArrays {
   uint32_t* episode;  // [N]
   uint32_t* nresets;  // [N]
   uint32_t* flags;    // [N] transient per-step bits, see kAgent*
-  float* geo;         // [N] result slot of the geodesic kernel
+  float* geo;         // [2N] geodesic results: [i] step query of agent i, [N + i] its reset query
   // outputs
   float* rewards;     // [N]
   uint8_t* masks;     // [N]
   float* infos;       // [N][3]
   float* polars;      // [N][2]
 };
-constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentNeedGeo = 4u, kAgentSkip = 8u;
+constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentSkip = 8u, kAgentResetOnly = 16u;
 
 struct NavData {
   const PolyRec* polys;
@@ -111,13 +117,11 @@ struct HeapEntry {
   uint32_t node;
 };
 
-// Scratch of one A* slot in HBM.
+// Spill area of one A* wavefront in HBM: nodes and open-list entries beyond what its LDS holds.
 struct alignas(128) GeoSlot {
   ANode nodes[kMaxNodes];
-  HeapEntry heap_spill[kMaxNodes];   // heap entries beyond the LDS-resident top
-  uint16_t next[kMaxNodes];          // hash chains
-  uint32_t corridor[kMaxPath];
-  float portals[kMaxPath][6];        // left xyz, right xyz of corridor portal i -> i+1
+  HeapEntry heap_spill[kMaxNodes];
+  uint16_t next[kMaxNodes];          // hash chains of the spilled nodes
 };
 
 struct GeoQuery {

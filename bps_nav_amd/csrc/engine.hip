@@ -25,8 +25,7 @@ using namespace bpsx;
 
 namespace {
 
-const char* const kKernelNames[BPSX_NUM_KERNELS] = {"step_move", "geodesic_step", "step_finish",
-                                                    "reset_snap", "geodesic_reset", "reset_finish"};
+const char* const kKernelNames[BPSX_NUM_KERNELS] = {"step_move", "reset_snap", "geodesic", "step_finish"};
 
 struct Group {
   StepQueues Q{};
@@ -64,7 +63,7 @@ struct bpsx_sim {
   std::vector<void*> owned;  // every device allocation, for destroy
   std::vector<Group> groups;
   GeoSlot* d_slots = nullptr;
-  uint32_t geo_blocks = 0;
+  uint32_t geo_blocks = 0, snap_blocks = 0;
   uint32_t* d_error = nullptr;
   uint64_t* d_counters = nullptr;
   float turn_left[4], turn_right[4];
@@ -87,6 +86,7 @@ struct bpsx_sim {
     StepParams P{};
     P.n = envs_per_group;
     P.base = group * envs_per_group;
+    P.total = cfg.num_environments;
     P.max_steps = (float)(cfg.max_steps ? cfg.max_steps : BPSX_MAX_STEPS);
     P.reset_mode = cfg.reset_mode;
     P.seed = cfg.seed;
@@ -190,7 +190,7 @@ int bpsx_finalize(bpsx_sim* sim) {
       (rc = sim->alloc(&A.goal_ref, N)) || (rc = sim->alloc(&A.prev_pos, N * 3)) || (rc = sim->alloc(&A.info_prev, N)) ||
       (rc = sim->alloc(&A.cum, N)) || (rc = sim->alloc(&A.init, N)) || (rc = sim->alloc(&A.rew_prev, N)) ||
       (rc = sim->alloc(&A.step, N)) || (rc = sim->alloc(&A.scene, N)) || (rc = sim->alloc(&A.episode, N)) ||
-      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.geo, N)) ||
+      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.geo, 2 * N)) ||
       (rc = sim->alloc(&A.rewards, N)) || (rc = sim->alloc(&A.masks, N)) || (rc = sim->alloc(&A.infos, N * 3)) ||
       (rc = sim->alloc(&A.polars, N * 2)))
     return rc;
@@ -207,25 +207,23 @@ int bpsx_finalize(bpsx_sim* sim) {
   if ((rc = sim->alloc(&sim->d_error, 1)) || (rc = sim->alloc(&sim->d_counters, BPSX_NUM_COUNTERS))) return rc;
   if ((rc = sim->alloc(&sim->d_batch_counts, 2))) return rc;
 
-  // ---- A* slots: a fixed pool sized by the device, not by the agent count
+  // ---- A* wavefronts: as many as the LDS of the device holds at once, not one per agent
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, sim->cfg.gpu_id));
-  uint32_t per_cu = 12;
-  if (const char* e = getenv("BPSX_GEO_BLOCKS_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e));
-  const uint32_t gpw = 64 / kGeoGroup;
+  uint32_t per_cu = 9;  // 160 KB of LDS per CU / 17 KB per A* wavefront
+  if (const char* e = getenv("BPSX_GEO_WAVES_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e));
   uint32_t blocks = (uint32_t)prop.multiProcessorCount * per_cu;
-  const uint32_t needed = (sim->envs_per_group + gpw - 1) / gpw;
-  if (blocks > needed) blocks = needed;
+  if (blocks > 2 * sim->envs_per_group) blocks = 2 * sim->envs_per_group;
   sim->geo_blocks = std::max(1u, blocks);
-  if ((rc = sim->alloc(&sim->d_slots, (size_t)sim->geo_blocks * gpw))) return rc;
+  sim->snap_blocks = std::max(1u, std::min((uint32_t)prop.multiProcessorCount * 16u, sim->envs_per_group));
+  if ((rc = sim->alloc(&sim->d_slots, (size_t)sim->geo_blocks))) return rc;
 
   // ---- per-group queues
   sim->groups.resize(sim->num_groups);
   const size_t n = sim->envs_per_group;
   for (auto& g : sim->groups) {
-    if ((rc = sim->alloc(&g.Q.counts, 8)) || (rc = sim->alloc(&g.Q.step_queries, n)) ||
-        (rc = sim->alloc(&g.Q.reset_queries, n)) || (rc = sim->alloc(&g.Q.reset_list, n)) ||
-        (rc = sim->alloc(&g.d_actions, n)))
+    if ((rc = sim->alloc(&g.Q.counts, 8)) || (rc = sim->alloc(&g.Q.queries, 2 * n)) ||
+        (rc = sim->alloc(&g.Q.reset_list, n)) || (rc = sim->alloc(&g.d_actions, n)))
       return rc;
     HIP_TRY(hipHostMalloc((void**)&g.h_actions, n * sizeof(int64_t), hipHostMallocDefault));
     HIP_TRY(hipEventCreateWithFlags(&g.done, hipEventDisableTiming));
@@ -272,7 +270,7 @@ int bpsx_reset(bpsx_sim* sim, uint32_t group, void* hip_stream) {
   if (g.in_flight) return fail(BPSX_E_STATE, "reset: a step of this group is still in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
   hipStream_t st = (hipStream_t)hip_stream;
-  launch_reset(sim->nav, sim->A, g.Q, sim->params(group), sim->d_slots, sim->geo_blocks, st);
+  launch_reset(sim->nav, sim->A, g.Q, sim->params(group), sim->d_slots, sim->geo_blocks, sim->snap_blocks, st);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipStreamSynchronize(st));
   return BPSX_OK;
@@ -295,7 +293,7 @@ int bpsx_step_start(bpsx_sim* sim, uint32_t group, const int64_t* actions, int a
     d_act = g.d_actions;
   }
   g.profiled = sim->profiling;
-  launch_step(sim->nav, sim->A, g.Q, sim->params(group), d_act, sim->d_slots, sim->geo_blocks, st,
+  launch_step(sim->nav, sim->A, g.Q, sim->params(group), d_act, sim->d_slots, sim->geo_blocks, sim->snap_blocks, st,
               g.profiled ? g.ev : nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipEventRecord(g.done, st));
@@ -414,7 +412,7 @@ int bpsx_snap_points(bpsx_sim* sim, uint32_t scene, const float* pts, uint32_t n
   char* b = (char*)sim->d_batch;
   float* d_in = (float*)b; float* d_xyz = (float*)(b + f3); uint32_t* d_ref = (uint32_t*)(b + 2 * f3);
   HIP_TRY(hipMemcpy(d_in, pts, f3, hipMemcpyHostToDevice));
-  launch_snap_batch(sim->nav, scene, d_in, n, d_xyz, d_ref, nullptr);
+  launch_snap_batch(sim->nav, scene, d_in, n, d_xyz, d_ref, sim->snap_blocks * 4, nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipMemcpy(out_xyz, d_xyz, f3, hipMemcpyDeviceToHost));
   HIP_TRY(hipMemcpy(out_ref, d_ref, (size_t)n * 4, hipMemcpyDeviceToHost));

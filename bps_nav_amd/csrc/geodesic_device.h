@@ -2,13 +2,15 @@
 // (string pulling) and the summed segment length, with the exact buffer limits and failure
 // conventions of the reference, so that the value equals PathFinder::findPath's.
 //
-// Execution model: a group of G consecutive lanes of one wavefront (G = 8, 16, 32 or 64)
-// owns one query at a time and pulls the next from a shared queue when done.  Inside a
-// group the sequential parts of A* (heap, node allocation order, funnel) run redundantly on
-// all lanes with lane 0 doing the stores; the per-edge work of a node expansion (neighbour
-// lookup in the node pool, portal midpoint, cost) is spread over the lanes.
-// The open list's top levels and the hash heads live in LDS, the node pool in a per-slot
-// scratch area in HBM.
+// Execution model: one wavefront (64 lanes) owns one query at a time and pulls the next from
+// a shared queue when done.  The whole working set of A* lives in LDS: the open list (a binary
+// heap whose pops and pushes are done by all lanes at once, see HeapOps), the hash heads and
+// chains of the node pool, and the first kNodesLds nodes; only nodes beyond that and heap
+// entries beyond kHeapLds spill to a per-wavefront scratch slot in HBM.  Per expanded node the
+// only HBM traffic is the polygon's 128-byte record.  Lane j of the wavefront handles edge j of
+// the expanded polygon (node lookup, portal midpoint, cost); heap updates are then applied in
+// edge order, which is what makes the result identical to the sequential algorithm, ties
+// included.
 //
 // Reference semantics followed: DetourNavMeshQuery.cpp:945-1178 (findPath, getPathToNode),
 // :1661-1696, 1765-1994 (appendVertex, findStraightPath), :2279-2349 (getPortalPoints);
@@ -18,208 +20,327 @@
 
 namespace bpsx {
 
-constexpr int kHeapLds = 256;   // open-list entries kept in LDS per group
+constexpr int kNodesLds = 512;   // nodes kept in LDS per query
+constexpr int kHeapLds = 512;    // open-list entries kept in LDS per query
 constexpr int kHashSize = 512;
 
-BPSX_DEV void group_sync() {
-  // Lanes of a group share a wavefront: ordering only has to be imposed on the compiler.
+BPSX_DEV void wave_sync() {
+  // All lanes belong to one wavefront: LDS and memory operations issue in program order, so
+  // only the compiler has to be kept from reordering across this point.
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   __builtin_amdgcn_wave_barrier();
 }
+BPSX_DEV int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
+BPSX_DEV float lane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
+BPSX_DEV int lane_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
 
-template <int G>
-BPSX_DEV uint32_t group_ballot(bool p, int grp) {
-  const unsigned long long m = __ballot(p);
-  if (G == 64) return 0;  // not used with 64 (callers use the 64-bit form)
-  return (uint32_t)((m >> (grp * G)) & ((1ull << G) - 1ull));
-}
+// LDS of one wavefront.
+struct GeoLds {
+  float n_total[kNodesLds];
+  float n_cost[kNodesLds];
+  float n_pos[3][kNodesLds];
+  uint32_t n_meta[kNodesLds];      // id:15 | flags:2 << 15 | pidx:12 << 17
+  uint16_t n_next[kNodesLds];
+  uint16_t first[kHashSize];
+  float h_total[kHeapLds];
+  uint16_t h_node[kHeapLds];
+};
+// After A* the node arrays are dead; the funnel reuses them for the corridor and its portals.
+struct FunnelLds {
+  float portals[kMaxPath][6];
+  uint16_t corridor[kMaxPath];
+};
+static_assert(sizeof(FunnelLds) <= offsetof(GeoLds, n_meta), "funnel scratch must stay clear of the node links");
 
-template <int G>
-struct GeoGroup {
-  HeapEntry* heap_lds;   // [kHeapLds]
-  uint16_t* first;       // [kHashSize]
+BPSX_DEV uint32_t meta_pack(uint32_t id, uint32_t flags, uint32_t pidx) { return id | (flags << 15) | (pidx << 17); }
+BPSX_DEV uint32_t meta_id(uint32_t m) { return m & 0x7fffu; }
+BPSX_DEV uint32_t meta_flags(uint32_t m) { return (m >> 15) & 3u; }
+BPSX_DEV uint32_t meta_pidx(uint32_t m) { return m >> 17; }
+
+struct NodeVal {
+  float pos[3];
+  float cost, total;
+  uint32_t meta;
+};
+
+struct GeoWave {
+  GeoLds* L;
   GeoSlot* ws;
-  int lane;              // 0..G-1
-  int grp;               // group index within the wavefront
+  int lane;
   int heapSize;
   int nodeCount;
 
-  BPSX_DEV unsigned long long gballot(bool p) const {
-    const unsigned long long m = __ballot(p);
-    if (G == 64) return m;
-    return (m >> (grp * G)) & ((1ull << G) - 1ull);
+  // ---------------------------------------------------------------- node pool
+  BPSX_DEV uint32_t node_meta(int i) const {
+    if (i < kNodesLds) return L->n_meta[i];
+    const ANode& n = ws->nodes[i];
+    return meta_pack(n.id, n.flags, n.pidx);
   }
-  BPSX_DEV HeapEntry hget(int i) const { return i < kHeapLds ? heap_lds[i] : ws->heap_spill[i]; }
-  BPSX_DEV void hset(int i, HeapEntry e) const {
-    if (lane == 0) {
-      if (i < kHeapLds) heap_lds[i] = e;
-      else ws->heap_spill[i] = e;
+  BPSX_DEV NodeVal node_load(int i) const {
+    NodeVal v;
+    if (i < kNodesLds) {
+      v.pos[0] = L->n_pos[0][i]; v.pos[1] = L->n_pos[1][i]; v.pos[2] = L->n_pos[2][i];
+      v.cost = L->n_cost[i]; v.total = L->n_total[i]; v.meta = L->n_meta[i];
+    } else {
+      const ANode n = ws->nodes[i];
+      v.pos[0] = n.pos[0]; v.pos[1] = n.pos[1]; v.pos[2] = n.pos[2];
+      v.cost = n.cost; v.total = n.total; v.meta = meta_pack(n.id, n.flags, n.pidx);
+    }
+    return v;
+  }
+  BPSX_DEV void node_store(int i, const NodeVal& v) const {
+    if (i < kNodesLds) {
+      L->n_pos[0][i] = v.pos[0]; L->n_pos[1][i] = v.pos[1]; L->n_pos[2][i] = v.pos[2];
+      L->n_cost[i] = v.cost; L->n_total[i] = v.total; L->n_meta[i] = v.meta;
+    } else {
+      ANode n;
+      n.pos[0] = v.pos[0]; n.pos[1] = v.pos[1]; n.pos[2] = v.pos[2];
+      n.cost = v.cost; n.total = v.total;
+      n.id = meta_id(v.meta); n.flags = meta_flags(v.meta); n.pidx = meta_pidx(v.meta);
+      ws->nodes[i] = n;
     }
   }
-  BPSX_DEV void bubble_up(int i, HeapEntry e) const {
-    int parent = (i - 1) / 2;
-    while (i > 0) {
-      const HeapEntry pe = hget(parent);
-      if (!(pe.total > e.total)) break;
-      hset(i, pe);
-      i = parent;
-      parent = (i - 1) / 2;
-    }
-    hset(i, e);
-    group_sync();
+  BPSX_DEV void node_set_meta(int i, uint32_t m) const {
+    if (i < kNodesLds) L->n_meta[i] = m;
+    else { ws->nodes[i].flags = meta_flags(m); ws->nodes[i].pidx = meta_pidx(m); ws->nodes[i].id = meta_id(m); }
   }
-  BPSX_DEV void trickle_down(int i, HeapEntry e) const {
-    int child = i * 2 + 1;
-    while (child < heapSize) {
-      HeapEntry c = hget(child);
-      if (child + 1 < heapSize) {
-        const HeapEntry c2 = hget(child + 1);
-        if (c.total > c2.total) { child++; c = c2; }
-      }
-      hset(i, c);
-      i = child;
-      child = i * 2 + 1;
-    }
-    group_sync();
-    bubble_up(i, e);
-  }
-  BPSX_DEV void push(HeapEntry e) {
-    heapSize++;
-    bubble_up(heapSize - 1, e);
-  }
-  BPSX_DEV HeapEntry pop() {
-    const HeapEntry r = hget(0);
-    heapSize--;
-    const HeapEntry last = hget(heapSize);
-    group_sync();
-    trickle_down(0, last);
-    return r;
-  }
-  // dtNodeQueue::modify: locate the node's entry (lanes scan in parallel), give it its new
-  // key and bubble it up from where it was.
-  BPSX_DEV void modify(uint32_t node, float total) const {
-    int found = -1;
-    for (int base = 0; base < heapSize; base += G) {
-      const int i = base + lane;
-      const bool hit = i < heapSize && hget(i).node == node;
-      const unsigned long long m = gballot(hit);
-      if (m) { found = base + (__ffsll((long long)m) - 1); break; }
-    }
-    if (found >= 0) bubble_up(found, HeapEntry{total, node});
-  }
+  BPSX_DEV int node_next(int i) const { return i < kNodesLds ? L->n_next[i] : ws->next[i]; }
   static BPSX_DEV uint32_t hash(uint32_t a) {
     a ^= a >> 16; a *= 0x7feb352du; a ^= a >> 15; a *= 0x846ca68bu; a ^= a >> 16;
     return a & (kHashSize - 1);
   }
   BPSX_DEV void clear() {
-    for (int i = lane; i < kHashSize; i += G) first[i] = 0xffff;
+    for (int i = lane; i < kHashSize; i += 64) L->first[i] = 0xffff;
     heapSize = 0;
     nodeCount = 0;
-    group_sync();
+    wave_sync();
   }
-  // node index of polygon `ip`, or -1
+  // node index of polygon ip, or -1 (any lane, independently)
   BPSX_DEV int find(uint32_t ip) const {
-    for (uint32_t i = first[hash(ip)]; i != 0xffff; i = ws->next[i])
-      if (ws->nodes[i].id == ip) return (int)i;
+    for (int i = L->first[hash(ip)]; i != 0xffff; i = node_next(i))
+      if (meta_id(node_meta(i)) == ip) return i;
     return -1;
   }
-  // Appends a node for `ip` (lane 0 writes); returns its index or -1 when the pool is full.
-  BPSX_DEV int alloc(uint32_t ip) {
-    if (nodeCount >= kMaxNodes) return -1;
-    const int i = nodeCount++;
+  // Links node i (already counted in nodeCount) into the hash; executed by one lane.
+  BPSX_DEV void link(int i, uint32_t ip) const {
     const uint32_t b = hash(ip);
-    if (lane == 0) {
-      ws->next[i] = first[b];
-      first[b] = (uint16_t)i;
-      ANode& n = ws->nodes[i];
-      n.pidx = 0; n.cost = 0; n.total = 0; n.id = ip; n.flags = 0;
+    const uint16_t head = L->first[b];
+    if (i < kNodesLds) L->n_next[i] = head;
+    else ws->next[i] = head;
+    L->first[b] = (uint16_t)i;
+  }
+
+  // ---------------------------------------------------------------- open list
+  BPSX_DEV float ht(int i) const { return i < kHeapLds ? L->h_total[i] : ws->heap_spill[i].total; }
+  BPSX_DEV int hn(int i) const { return i < kHeapLds ? (int)L->h_node[i] : (int)ws->heap_spill[i].node; }
+  BPSX_DEV void hset(int i, float t, int n) const {
+    if (i < kHeapLds) { L->h_total[i] = t; L->h_node[i] = (uint16_t)n; }
+    else { ws->heap_spill[i].total = t; ws->heap_spill[i].node = (uint32_t)n; }
+  }
+  // dtNodeQueue::bubbleUp from index i0 with entry (t, n), all ancestors looked at at once:
+  // along a leaf-to-root path the keys never increase, so the ancestors that are greater than
+  // t form a prefix; they each move one level down and the entry lands above them.
+  BPSX_DEV void bubble_up(int i0, float t, int n) const {
+    // lane d holds ancestor a_d = ((i0 + 1) >> d) - 1 (a_0 = i0; -1 once past the root)
+    const int a = lane <= 12 ? ((i0 + 1) >> lane) - 1 : -1;
+    const bool valid = lane >= 1 && a >= 0;
+    float at = 0;
+    int an = 0;
+    if (valid) { at = ht(a); an = hn(a); }
+    const unsigned long long gt = __ballot(valid && at > t);
+    const int m = __popcll(gt);  // ancestors 1..m move down
+    wave_sync();
+    // lane d (1..m) writes its ancestor's entry one level down, into a_{d-1}
+    const int child = lane >= 1 && lane <= 13 ? ((i0 + 1) >> (lane - 1)) - 1 : 0;
+    if (lane >= 1 && lane <= m) hset(child, at, an);
+    if (lane == m) hset(lane == 0 ? i0 : a, t, n);
+    wave_sync();
+  }
+  BPSX_DEV void push(float t, int n) {
+    heapSize++;
+    bubble_up(heapSize - 1, t, n);
+  }
+  BPSX_DEV void modify(int n, float t) const {
+    int found = -1;
+    for (int base = 0; base < heapSize; base += 64) {
+      const int i = base + lane;
+      const unsigned long long m = __ballot(i < heapSize && hn(i) == n);
+      if (m) { found = base + (__ffsll((long long)m) - 1); break; }
     }
-    group_sync();
-    return i;
+    if (found >= 0) bubble_up(found, t, n);
+  }
+  // dtNodeQueue::pop: the hole left by the root travels down along the smaller children to a
+  // leaf, then the former last entry bubbles up from there.  The route depends only on the
+  // heap's contents, so lanes evaluate "which child is smaller" for 63 nodes of a subtree at
+  // once and the route is then read off with scalar lane reads; the entries on the route that
+  // are not greater than the re-inserted entry shift up one level, it lands below them, and
+  // the rest of the route stays as it was.
+  BPSX_DEV int pop() {
+    const int top = hn(0);
+    heapSize--;
+    const int size = heapSize;
+    if (size == 0) return top;
+    const float lt = ht(size);
+    const int ln = hn(size);
+    // route entries are collected one per lane: lane d keeps the d-th node of the route
+    float myT = 0;
+    int myN = 0, myIdx = -1, myParent = -1;
+    int depth = 0;   // number of route nodes below the root found so far (uniform)
+    int root = 0;    // root of the subtree being resolved (uniform)
+    for (;;) {
+      // lane t (< 63) looks at node (root+1 << lvl) - 1 + off of the subtree, lvl = floor(log2(t+1))
+      const int t1 = lane + 1;
+      const int lvl = 31 - __clz(t1);
+      const int node = ((root + 1) << lvl) - 1 + (t1 - (1 << lvl));
+      int choice = -1;
+      float ct = 0;
+      int cn = 0;
+      if (lane < 63) {
+        const int c1 = 2 * node + 1;
+        if (c1 < size && node < size) {
+          ct = ht(c1); cn = hn(c1); choice = c1;
+          if (c1 + 1 < size) {
+            const float t2 = ht(c1 + 1);
+            if (ct > t2) { ct = t2; cn = hn(c1 + 1); choice = c1 + 1; }
+          }
+        }
+      }
+      // follow the choices from the subtree's root: relative lane r -> 2r+1 or 2r+2
+      int r = 0, cur = root;
+      bool more = false;
+      for (int s = 0; s < 6; ++s) {
+        const int c = lane_i(choice, r);
+        if (c < 0) break;
+        const float tt = lane_f(ct, r);
+        const int nn = lane_i(cn, r);
+        depth++;
+        if (lane == depth) { myT = tt; myN = nn; myIdx = c; myParent = cur; }
+        r = 2 * r + 1 + (c - (2 * cur + 1));
+        cur = c;
+        if (r >= 63) { more = true; break; }
+      }
+      if (!more) break;
+      root = cur;
+    }
+    const unsigned long long le = __ballot(lane >= 1 && lane <= depth && myT <= lt);
+    const int j = __popcll(le);  // route entries 1..j shift up, the re-inserted entry lands at route[j]
+    wave_sync();
+    if (lane >= 1 && lane <= j) hset(myParent, myT, myN);
+    if (lane == j) hset(j == 0 ? 0 : myIdx, lt, ln);
+    wave_sync();
+    return top;
   }
 };
 
-template <int G>
-BPSX_DEV float bcast_f(float v, int src) { return __shfl(v, src, G); }
-template <int G>
-BPSX_DEV int bcast_i(int v, int src) { return __shfl(v, src, G); }
-
-// Runs A* for one query. Returns the corridor length written to ws->corridor, or 0 when the
-// reference would report anything but plain DT_SUCCESS.
-template <int G>
-BPSX_DEV int astar(GeoGroup<G>& g, const NavData& nav, const SceneDev& s, uint32_t startIp, uint32_t endIp,
+// Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
+// when the reference would report anything but plain DT_SUCCESS.
+BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev& s, uint32_t startIp, uint32_t endIp,
                    const float* startPos, const float* endPos, uint32_t* pops) {
   const int lane = g.lane;
-  GeoSlot* ws = g.ws;
   if (startIp == endIp) {
-    if (lane == 0) ws->corridor[0] = startIp;
-    group_sync();
+    if (lane == 0) F->corridor[0] = (uint16_t)startIp;
+    wave_sync();
     return 1;
   }
   g.clear();
   const float H_SCALE = 0.999f;
   {
-    const int si = g.alloc(startIp);
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
     const float total = sqrtf(dx * dx + dy * dy + dz * dz) * H_SCALE;
+    g.nodeCount = 1;
     if (lane == 0) {
-      ANode& n = ws->nodes[si];
-      n.pos[0] = startPos[0]; n.pos[1] = startPos[1]; n.pos[2] = startPos[2];
-      n.pidx = 0; n.cost = 0; n.total = total; n.id = startIp; n.flags = 1;
+      NodeVal v;
+      v.pos[0] = startPos[0]; v.pos[1] = startPos[1]; v.pos[2] = startPos[2];
+      v.cost = 0; v.total = total; v.meta = meta_pack(startIp, 1u, 0u);
+      g.node_store(0, v);
+      g.link(0, startIp);
     }
-    group_sync();
-    g.push(HeapEntry{total, (uint32_t)si});
+    wave_sync();
+    g.push(total, 0);
   }
   int lastBest = 0;
-  float lastBestCost = ws->nodes[0].total;
+  float lastBestCost = g.L->n_total[0];
   bool outOfNodes = false;
   while (g.heapSize > 0) {
-    const HeapEntry top = g.pop();
-    const int bi = (int)top.node;
-    const ANode best = ws->nodes[bi];
-    if (lane == 0) ws->nodes[bi].flags = (best.flags & ~1u) | 2u;
-    group_sync();
-    if (best.id == endIp) { lastBest = bi; break; }
+    // the node about to be popped is the root: fetch its polygon while the heap is repaired
+    const int bi = uniform_i(g.hn(0));
+    const NodeVal best = g.node_load(bi);
+    const uint32_t bestIp = meta_id(best.meta);
+    const PolyRec* bp = &nav.polys[s.poly_base + bestIp];
+    uint32_t nbRaw = 0, nbWalk = 0;
+    float l0 = 0, l1 = 0, l2 = 0, r0 = 0, r1 = 0, r2 = 0;
+    const int nv = bp->nv;
+    if (lane < kNvp) {
+      nbRaw = bp->nei[lane];
+      nbWalk = bp->walk[lane];
+      l0 = bp->v[lane][0]; l1 = bp->v[lane][1]; l2 = bp->v[lane][2];
+    }
+    const uint32_t pidx = meta_pidx(best.meta);
+    const uint32_t parentIp = pidx ? meta_id(g.node_meta((int)pidx - 1)) : kInvalidPoly;
+    g.pop();
+    if (lane == 0) g.node_set_meta(bi, meta_pack(bestIp, (meta_flags(best.meta) & ~1u) | 2u, pidx));
+    wave_sync();
+    if (bestIp == endIp) { lastBest = bi; break; }
     (*pops)++;
-    const PolyRec& bp = nav.polys[s.poly_base + best.id];
-    const uint32_t parentIp = best.pidx ? ws->nodes[best.pidx - 1].id : kInvalidPoly;
+    // right end of edge j is the left end of edge j+1 (mod nv)
+    {
+      const int nxt = lane + 1 < nv ? lane + 1 : 0;
+      r0 = __shfl(l0, nxt); r1 = __shfl(l1, nxt); r2 = __shfl(l2, nxt);
+    }
     // ---- per-edge phase: lane j looks at edge j
-    const int nv = bp.nv;
     uint32_t nb = kInvalidPoly;
     if (lane < nv) {
-      const uint16_t w = (bp.nei[lane] & 0x8000) ? (uint16_t)0 : bp.nei[lane];
-      // the link exists for every internal edge; the filter is applied to the neighbour
-      if (w && (uint32_t)(w - 1) != parentIp && bp.walk[lane]) nb = (uint32_t)(w - 1);
+      const uint32_t w = (nbRaw & 0x8000u) ? 0u : nbRaw;
+      if (w && (w - 1) != parentIp && nbWalk) nb = w - 1;
     }
     // a polygon reached through two edges of the same expansion: the second visit never
     // changes the node (same position, same cost), so only the first edge counts
+#pragma unroll
     for (int k = 0; k < kNvp - 1; ++k) {
-      const uint32_t other = (uint32_t)bcast_i<G>((int)nb, k);
+      const uint32_t other = (uint32_t)__shfl((int)nb, k);
       if (lane > k && nb != kInvalidPoly && other == nb) nb = kInvalidPoly;
     }
     int ni = -1;
     if (nb != kInvalidPoly) ni = g.find(nb);
-    // allocation in edge order (the pool may run out part-way)
-    unsigned long long need = g.gballot(nb != kInvalidPoly && ni < 0);
-    while (need) {
-      const int src = __ffsll((long long)need) - 1;
-      need &= need - 1;
-      const uint32_t ip = (uint32_t)bcast_i<G>((int)nb, src);
-      const int idx = g.alloc(ip);
-      if (idx < 0) outOfNodes = true;
-      if (lane == src) { ni = idx; if (idx < 0) nb = kInvalidPoly; }
+    // new nodes take consecutive indices in edge order; past the pool's end they are dropped
+    {
+      const unsigned long long need = __ballot(nb != kInvalidPoly && ni < 0);
+      if (need) {
+        const int rank = __popcll(need & ((1ull << lane) - 1ull));
+        const bool mine = (need >> lane) & 1ull;
+        if (mine) {
+          const int idx = g.nodeCount + rank;
+          if (idx < kMaxNodes) ni = idx;
+          else nb = kInvalidPoly;
+        }
+        const int want = g.nodeCount + __popcll(need);
+        if (want > kMaxNodes) outOfNodes = true;
+        g.nodeCount = want < kMaxNodes ? want : kMaxNodes;
+        // hash insertion one node at a time (two new nodes may share a bucket)
+        unsigned long long todo = need;
+        while (todo) {
+          const int src = __ffsll((long long)todo) - 1;
+          todo &= todo - 1;
+          if (lane == src && nb != kInvalidPoly) g.link(ni, nb);
+          wave_sync();
+        }
+        if (mine && nb != kInvalidPoly) {
+          NodeVal v;
+          v.pos[0] = v.pos[1] = v.pos[2] = 0; v.cost = 0; v.total = 0; v.meta = meta_pack(nb, 0u, 0u);
+          g.node_store(ni, v);
+        }
+      }
     }
     bool update = false;
     float total = 0, heuristic = 0;
     bool wasOpen = false;
     if (nb != kInvalidPoly) {
-      ANode nn = ws->nodes[ni];
-      if (nn.flags == 0) {
-        const float* l = bp.v[lane];
-        const float* r = bp.v[(lane + 1) % nv];
-        nn.pos[0] = (l[0] + r[0]) * 0.5f;
-        nn.pos[1] = (l[1] + r[1]) * 0.5f;
-        nn.pos[2] = (l[2] + r[2]) * 0.5f;
+      NodeVal nn = g.node_load(ni);
+      uint32_t fl = meta_flags(nn.meta);
+      if (fl == 0) {
+        nn.pos[0] = (l0 + r0) * 0.5f;
+        nn.pos[1] = (l1 + r1) * 0.5f;
+        nn.pos[2] = (l2 + r2) * 0.5f;
       }
       const float cx = nn.pos[0] - best.pos[0], cy = nn.pos[1] - best.pos[1], cz = nn.pos[2] - best.pos[2];
       const float curCost = sqrtf(cx * cx + cy * cy + cz * cz) * 1.0f;
@@ -234,46 +355,47 @@ BPSX_DEV int astar(GeoGroup<G>& g, const NavData& nav, const SceneDev& s, uint32
         heuristic = toEnd * H_SCALE;
       }
       total = cost + heuristic;
-      const bool worse = (nn.flags & 3u) && total >= nn.total;
+      const bool worse = (fl & 3u) && total >= nn.total;
       if (!worse) {
         update = true;
-        wasOpen = (nn.flags & 1u) != 0;
-        nn.pidx = (uint32_t)bi + 1;
-        nn.id = nb;
-        nn.flags = (nn.flags & ~2u) | 1u;
+        wasOpen = (fl & 1u) != 0;
+        nn.meta = meta_pack(nb, (fl & ~2u) | 1u, (uint32_t)bi + 1);
         nn.cost = cost;
         nn.total = total;
-        ws->nodes[ni] = nn;
+        g.node_store(ni, nn);
       }
     }
-    group_sync();
+    wave_sync();
     // ---- ordered phase: heap and "nearest so far" updates in edge order
-    unsigned long long upd = g.gballot(update);
+    unsigned long long upd = __ballot(update);
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
-      const int node = bcast_i<G>(ni, src);
-      const float t = bcast_f<G>(total, src);
-      const float h = bcast_f<G>(heuristic, src);
-      const bool open = bcast_i<G>(wasOpen ? 1 : 0, src) != 0;
-      if (open) g.modify((uint32_t)node, t);
-      else g.push(HeapEntry{t, (uint32_t)node});
+      const int node = lane_i(ni, src);
+      const float t = lane_f(total, src);
+      const float h = lane_f(heuristic, src);
+      const bool open = lane_i(wasOpen ? 1 : 0, src) != 0;
+      if (open) g.modify(node, t);
+      else g.push(t, node);
       if (h < lastBestCost) { lastBestCost = h; lastBest = node; }
     }
   }
   // getPathToNode
   int length = 0;
-  for (int c = lastBest + 1; c; c = (int)ws->nodes[c - 1].pidx) length++;
-  const bool ok = length <= kMaxPath && ws->nodes[lastBest].id == endIp && !outOfNodes;
+  for (int c = lastBest + 1; c; c = (int)meta_pidx(g.node_meta(c - 1))) length++;
+  const bool ok = length <= kMaxPath && meta_id(g.node_meta(lastBest)) == endIp && !outOfNodes;
   if (!ok) return 0;
+  // the corridor goes into LDS that overlays the nodes' cost and position arrays; the parent
+  // links (n_meta) are outside that region and stay readable while it is written
   if (lane == 0) {
     int c = lastBest + 1;
     for (int i = length - 1; i >= 0; --i) {
-      ws->corridor[i] = ws->nodes[c - 1].id;
-      c = (int)ws->nodes[c - 1].pidx;
+      const uint32_t m = g.node_meta(c - 1);
+      F->corridor[i] = (uint16_t)meta_id(m);
+      c = (int)meta_pidx(m);
     }
   }
-  group_sync();
+  wave_sync();
   return length;
 }
 
@@ -288,32 +410,30 @@ BPSX_DEV bool vequal(const float* a, const float* b) {
   return dx * dx + dy * dy + dz * dz < thr;
 }
 
-// String pulling over ws->corridor[0..n) and the summed length; +inf for every outcome the
+// String pulling over F->corridor[0..n) and the summed length; +inf for every outcome the
 // reference maps to "no path" (straight path of 256 points or more, missing portal).
-template <int G>
-BPSX_DEV float funnel_length(GeoGroup<G>& g, const NavData& nav, const SceneDev& s, int n, const float* startPos,
+BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const SceneDev& s, int n, const float* startPos,
                              const float* endPos) {
-  GeoSlot* ws = g.ws;
   const float INF = __int_as_float(0x7f800000);
-  // gather the portals of the corridor, G at a time
+  // gather the portals of the corridor, 64 at a time
   bool missing = false;
-  for (int i = g.lane; i + 1 < n; i += G) {
-    const PolyRec& r = nav.polys[s.poly_base + ws->corridor[i]];
-    const uint32_t to = ws->corridor[i + 1];
+  for (int i = lane; i + 1 < n; i += 64) {
+    const PolyRec& r = nav.polys[s.poly_base + F->corridor[i]];
+    const uint32_t to = F->corridor[i + 1];
     int e = -1;
     for (int k = 0; k < r.nv; ++k)
       if (r.nei[k] && !(r.nei[k] & 0x8000) && (uint32_t)(r.nei[k] - 1) == to) { e = k; break; }
     if (e < 0) { missing = true; continue; }
     const float* l = r.v[e];
     const float* rr = r.v[(e + 1) % r.nv];
-    float* p = ws->portals[i];
+    float* p = F->portals[i];
     p[0] = l[0]; p[1] = l[1]; p[2] = l[2]; p[3] = rr[0]; p[4] = rr[1]; p[5] = rr[2];
   }
-  group_sync();
-  if (g.gballot(missing)) return INF;
+  wave_sync();
+  if (__ballot(missing)) return INF;
   float cs[3], ce[3];
-  closest_on_poly_boundary(nav.polys[s.poly_base + ws->corridor[0]], startPos, cs);
-  closest_on_poly_boundary(nav.polys[s.poly_base + ws->corridor[n - 1]], endPos, ce);
+  closest_on_poly_boundary(nav.polys[s.poly_base + F->corridor[0]], startPos, cs);
+  closest_on_poly_boundary(nav.polys[s.poly_base + F->corridor[n - 1]], endPos, ce);
   // straight-path points are only needed pairwise: keep the last one and the running length
   float last[3] = {cs[0], cs[1], cs[2]};
   int npts = 1;
@@ -335,7 +455,7 @@ BPSX_DEV float funnel_length(GeoGroup<G>& g, const NavData& nav, const SceneDev&
     for (int i = 0; i < n && !finished; ++i) {
       float left[3], right[3];
       if (i + 1 < n) {
-        const float* p = ws->portals[i];
+        const float* p = F->portals[i];
         left[0] = p[0]; left[1] = p[1]; left[2] = p[2];
         right[0] = p[3]; right[1] = p[4]; right[2] = p[5];
         if (i == 0) {
@@ -386,9 +506,8 @@ BPSX_DEV float funnel_length(GeoGroup<G>& g, const NavData& nav, const SceneDev&
   return overflow ? INF : length;
 }
 
-// Full PathFinder::findPath distance for one query, executed by a group.
-template <int G>
-BPSX_DEV float geodesic_query(GeoGroup<G>& g, const NavData& nav, const GeoQuery& q, uint32_t* pops, uint32_t* corridor) {
+// Full PathFinder::findPath distance for one query, executed by a wavefront.
+BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q, uint32_t* pops, uint32_t* corridor) {
   const float INF = __int_as_float(0x7f800000);
   {
     // Eigen isApprox with default precision; sums of three reduce as a0 + (a1 + a2)
@@ -405,10 +524,11 @@ BPSX_DEV float geodesic_query(GeoGroup<G>& g, const NavData& nav, const GeoQuery
   if (sIp == kInvalidPoly || eIp == kInvalidPoly) return INF;
   if (nav.polys[s.poly_base + sIp].island != nav.polys[s.poly_base + eIp].island) return INF;
   if (!finite3(q.a[0], q.a[1], q.a[2]) || !finite3(q.b[0], q.b[1], q.b[2])) return INF;
-  const int n = astar<G>(g, nav, s, sIp, eIp, q.a, q.b, pops);
+  FunnelLds* F = reinterpret_cast<FunnelLds*>(g.L);
+  const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops);
   if (n <= 0) return INF;
   *corridor += (uint32_t)n;
-  return funnel_length<G>(g, nav, s, n, q.a, q.b);
+  return funnel_length(g.lane, F, nav, s, n, q.a, q.b);
 }
 
 }  // namespace bpsx

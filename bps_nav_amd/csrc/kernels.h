@@ -6,21 +6,19 @@
 
 namespace bpsx {
 
-constexpr int kGeoGroup = 16;  // lanes that cooperate on one geodesic query
-
-enum QueueCounter { kQStepGeo = 0, kQStepGeoHead, kQReset, kQResetGeo, kQResetGeoHead, kQSpare };
+enum QueueCounter { kQGeo = 0, kQGeoHead, kQReset };
 
 // Work queues of one step, all in HBM, sized for every agent of a group.
 struct StepQueues {
-  uint32_t* counts;          // [6], see QueueCounter
-  GeoQuery* step_queries;    // [n]
-  GeoQuery* reset_queries;   // [n]
+  uint32_t* counts;          // [4], see QueueCounter
+  GeoQuery* queries;         // [2n]: one per moved/finished agent plus one per reset
   uint32_t* reset_list;      // [n] agent indices being reset
 };
 
 struct StepParams {
   uint32_t n;          // agents in the group
   uint32_t base;       // index of the group's first agent
+  uint32_t total;      // agents in the simulator (reset results live at geo[total + i])
   float max_steps;
   uint32_t reset_mode;
   uint64_t seed;
@@ -29,14 +27,15 @@ struct StepParams {
   uint64_t* counters;
 };
 
-constexpr int kStepEvents = 7;  // timestamps recorded by launch_step when asked to
+constexpr int kStepEvents = 5;  // timestamps recorded by launch_step when asked to
 
 void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
-                 const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, hipStream_t st, hipEvent_t* ev);
+                 const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st,
+                 hipEvent_t* ev);
 void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P, GeoSlot* slots,
-                  uint32_t geo_blocks, hipStream_t st);
+                  uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st);
 void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref,
-                       hipStream_t st);
+                       uint32_t snap_blocks, hipStream_t st);
 void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
                            uint32_t n, float* oxyz, uint32_t* oref, hipStream_t st);
 void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,

@@ -1,16 +1,17 @@
 // HIP kernels of the batch environment step (gfx950) and their launch wrappers.
 //
-// One step of a group of n agents is six launches on one stream:
+// One step of a group of n agents is four launches on one stream:
 //   step_move      lane per agent: action, turn / forward move with wall sliding, polar
 //                  observation, and a geodesic query (goal -> agent) when the agent moved or
-//                  the episode ended                     (simulator.cpp:620-632, 651-710)
-//   geodesic       group of lanes per query: A* + funnel (PathFinder.cpp:485-541)
-//   step_finish    lane per agent: info, reward, mask; a finished episode picks its next
-//                  episode and is queued for reset      (simulator.cpp:634-641, 758-822, 601-610)
-//   reset_snap     lane per queued agent: snap start and goal, polar, query (agent -> goal)
+//                  the episode ended; an agent whose episode ended also picks its next episode
+//                  here and is queued for reset (simulator.cpp:620-632, 651-710, 601-610)
+//   reset_snap     wavefront per queued agent: snap start and goal of the new episode, polar,
+//                  and the new episode's first query (agent -> goal)
 //                                                        (simulator.cpp:611-614, 744-751)
-//   geodesic       the reset queries
-//   reset_finish   lane per queued agent: initial distance bookkeeping (simulator.cpp:749-755, 801-806)
+//   geodesic       wavefront per query, both kinds in one launch: A* + funnel
+//                                                        (PathFinder.cpp:485-541)
+//   step_finish    lane per agent: info, reward, mask from the terminal transition, then the
+//                  new episode's distance bookkeeping    (simulator.cpp:634-641, 758-822, 749-755)
 #include <hip/hip_runtime.h>
 
 #include "geodesic_device.h"
@@ -86,18 +87,49 @@ BPSX_DEV void store3(float* p, size_t i, const float* v) { p[i * 3] = v[0]; p[i 
 
 __global__ void k_clear_queues(StepQueues Q) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
-    Q.counts[0] = 0; Q.counts[1] = 0; Q.counts[2] = 0; Q.counts[3] = 0; Q.counts[4] = 0; Q.counts[5] = 0;
+    Q.counts[kQGeo] = 0; Q.counts[kQGeoHead] = 0; Q.counts[kQReset] = 0;
   }
+}
+
+// Picks the next episode of agent gi and writes its pose; the snaps follow in reset_snap.
+BPSX_DEV void begin_reset(const NavData& nav, const AgentArrays& A, const StepParams& P, uint32_t gi) {
+  const uint32_t count = A.nresets[gi];
+  A.nresets[gi] = count + 1;
+  A.step[gi] = 1;
+  const uint32_t sc = A.scene[gi];
+  const SceneDev& s = nav.scenes[sc];
+  const uint64_t key = reset_key(P.seed, gi, count);
+  float ep[10];
+  if (P.reset_mode == 0) {
+    const uint32_t e = draw_index(reset_draw(key, 0), s.ep_count);
+    A.episode[gi] = e;
+    for (int k = 0; k < 10; ++k) ep[k] = nav.episodes[(size_t)(s.ep_base + e) * 10 + k];
+  } else {
+    A.episode[gi] = 0;
+    float a[3] = {0, 0, 0}, b[3] = {0, 0, 0};
+    uint32_t ip;
+    sample_point(nav, s, draw_unit(reset_draw(key, 0)), draw_unit(reset_draw(key, 1)), draw_unit(reset_draw(key, 2)), a, &ip);
+    sample_point(nav, s, draw_unit(reset_draw(key, 3)), draw_unit(reset_draw(key, 4)), draw_unit(reset_draw(key, 5)), b, &ip);
+    const uint32_t turns = draw_index(reset_draw(key, 6), 36);
+    float q[4] = {0, 0, 0, 1};
+    for (uint32_t t = 0; t < turns; ++t) quat_mul(q, P.turn_left, q);
+    ep[0] = a[0]; ep[1] = a[1]; ep[2] = a[2];
+    ep[3] = q[0]; ep[4] = q[1]; ep[5] = q[2]; ep[6] = q[3];
+    ep[7] = b[0]; ep[8] = b[1]; ep[9] = b[2];
+  }
+  store3(A.pos, gi, ep);
+  for (int k = 0; k < 4; ++k) A.rot[(size_t)gi * 4 + k] = ep[3 + k];
+  store3(A.goal, gi, ep + 7);
 }
 
 __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, StepQueues Q, StepParams P,
                                                    const int64_t* __restrict__ actions) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  bool want = false;
+  bool want = false, reset = false;
   GeoQuery q{};
-  uint32_t movePolys = 0;
+  uint32_t movePolys = 0, gi = 0;
   if (i < P.n) {
-    const uint32_t gi = P.base + i;
+    gi = P.base + i;
     const int64_t action = actions[i];
     if (action < 0 || action > 3) {
       // the reference aborts here (simulator.cpp:704-708); flag it and leave the agent alone
@@ -145,10 +177,18 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         q.scene = A.scene[gi];
         q.out = gi;
       }
+      if (done) {
+        // the terminal query above holds copies of the old episode's points: the pose arrays can
+        // take the next episode now; distance bookkeeping waits for step_finish
+        begin_reset(nav, A, P, gi);
+        reset = true;
+      }
     }
   }
-  const uint32_t slot = wave_append(want, &Q.counts[kQStepGeo]);
-  if (want) Q.step_queries[slot] = q;
+  const uint32_t slot = wave_append(want, &Q.counts[kQGeo]);
+  if (want) Q.queries[slot] = q;
+  const uint32_t rslot = wave_append(reset, &Q.counts[kQReset]);
+  if (reset) Q.reset_list[rslot] = gi;
   // counters, one atomic per wavefront
   const unsigned long long mv = __ballot(movePolys != 0);
   uint32_t mp = movePolys;
@@ -162,82 +202,54 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
   if (i == 0) atomicAdd((unsigned long long*)&P.counters[kCntSteps], (unsigned long long)P.n);
 }
 
-// Picks the next episode of agent gi and writes its pose; the snaps follow in reset_snap.
-BPSX_DEV void begin_reset(const NavData& nav, const AgentArrays& A, const StepParams& P, uint32_t gi) {
-  const uint32_t count = A.nresets[gi];
-  A.nresets[gi] = count + 1;
-  A.step[gi] = 1;
-  const uint32_t sc = A.scene[gi];
-  const SceneDev& s = nav.scenes[sc];
-  const uint64_t key = reset_key(P.seed, gi, count);
-  float ep[10];
-  if (P.reset_mode == 0) {
-    const uint32_t e = draw_index(reset_draw(key, 0), s.ep_count);
-    A.episode[gi] = e;
-    for (int k = 0; k < 10; ++k) ep[k] = nav.episodes[(size_t)(s.ep_base + e) * 10 + k];
-  } else {
-    A.episode[gi] = 0;
-    float a[3] = {0, 0, 0}, b[3] = {0, 0, 0};
-    uint32_t ip;
-    sample_point(nav, s, draw_unit(reset_draw(key, 0)), draw_unit(reset_draw(key, 1)), draw_unit(reset_draw(key, 2)), a, &ip);
-    sample_point(nav, s, draw_unit(reset_draw(key, 3)), draw_unit(reset_draw(key, 4)), draw_unit(reset_draw(key, 5)), b, &ip);
-    const uint32_t turns = draw_index(reset_draw(key, 6), 36);
-    float q[4] = {0, 0, 0, 1};
-    for (uint32_t t = 0; t < turns; ++t) quat_mul(q, P.turn_left, q);
-    ep[0] = a[0]; ep[1] = a[1]; ep[2] = a[2];
-    ep[3] = q[0]; ep[4] = q[1]; ep[5] = q[2]; ep[6] = q[3];
-    ep[7] = b[0]; ep[8] = b[1]; ep[9] = b[2];
-  }
-  store3(A.pos, gi, ep);
-  for (int k = 0; k < 4; ++k) A.rot[(size_t)gi * 4 + k] = ep[3 + k];
-  store3(A.goal, gi, ep + 7);
-}
-
-__global__ __launch_bounds__(256) void k_step_finish(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
+__global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  bool reset = false;
-  uint32_t gi = 0;
-  if (i < P.n) {
-    gi = P.base + i;
-    const uint32_t f = A.flags[gi];
-    if (!(f & kAgentSkip)) {
-      const bool done = f & kAgentDone, moved = f & kAgentMoved;
-      float dist, success = 0, spl = 0;
-      if (done) {
-        dist = A.geo[gi];
-        success = dist < 0.2f ? 1.0f : 0.0f;
-        const float init = A.init[gi], cum = A.cum[gi];
-        const float mx = init < cum ? cum : init;
-        spl = success * init / mx;
-      } else if (moved) {
-        dist = A.geo[gi];
-        float pos[3], pp[3];
-        load3(A.pos, gi, pos);
-        load3(A.prev_pos, gi, pp);
-        const float dx = pos[0] - pp[0], dy = pos[1] - pp[1], dz = pos[2] - pp[2];
-        A.cum[gi] = A.cum[gi] + sqrtf(dx * dx + dy * dy + dz * dz);
-        A.info_prev[gi] = dist;
-        store3(A.prev_pos, gi, pos);
-      } else {
-        dist = A.info_prev[gi];
-      }
-      float reward = -1e-2f;
-      if (done) reward += 2.5f * spl;
-      else reward += A.rew_prev[gi] - dist;
-      A.rew_prev[gi] = dist;
-      A.rewards[gi] = reward;
-      A.masks[gi] = done ? 0 : 1;
-      A.infos[(size_t)gi * 3 + 0] = success;
-      A.infos[(size_t)gi * 3 + 1] = spl;
-      A.infos[(size_t)gi * 3 + 2] = dist;
-      if (done) {
-        begin_reset(nav, A, P, gi);
-        reset = true;
-      }
+  if (i >= P.n) return;
+  const uint32_t gi = P.base + i;
+  const uint32_t f = A.flags[gi];
+  if (f & kAgentSkip) return;
+  const bool done = f & kAgentDone, moved = f & kAgentMoved;
+  if (!(f & kAgentResetOnly)) {
+    float dist, success = 0, spl = 0;
+    if (done) {
+      dist = A.geo[gi];
+      success = dist < 0.2f ? 1.0f : 0.0f;
+      const float init = A.init[gi], cum = A.cum[gi];
+      const float mx = init < cum ? cum : init;
+      spl = success * init / mx;
+    } else if (moved) {
+      dist = A.geo[gi];
+      float pos[3], pp[3];
+      load3(A.pos, gi, pos);
+      load3(A.prev_pos, gi, pp);
+      const float dx = pos[0] - pp[0], dy = pos[1] - pp[1], dz = pos[2] - pp[2];
+      A.cum[gi] = A.cum[gi] + sqrtf(dx * dx + dy * dy + dz * dz);
+      A.info_prev[gi] = dist;
+      store3(A.prev_pos, gi, pos);
+    } else {
+      dist = A.info_prev[gi];
     }
+    float reward = -1e-2f;
+    if (done) reward += 2.5f * spl;
+    else reward += A.rew_prev[gi] - dist;
+    A.rew_prev[gi] = dist;
+    A.rewards[gi] = reward;
+    A.masks[gi] = done ? 0 : 1;
+    A.infos[(size_t)gi * 3 + 0] = success;
+    A.infos[(size_t)gi * 3 + 1] = spl;
+    A.infos[(size_t)gi * 3 + 2] = dist;
   }
-  const uint32_t slot = wave_append(reset, &Q.counts[kQReset]);
-  if (reset) Q.reset_list[slot] = gi;
+  if (done || (f & kAgentResetOnly)) {
+    // InfoFunctor::reset / RewardFunctor::reset with the new episode's first distance
+    const float d = A.geo[(size_t)P.total + gi];
+    A.cum[gi] = 0;
+    A.init[gi] = d;
+    A.info_prev[gi] = d;
+    A.rew_prev[gi] = d;
+    float pos[3];
+    load3(A.pos, gi, pos);
+    store3(A.prev_pos, gi, pos);
+  }
 }
 
 __global__ __launch_bounds__(256) void k_reset_all(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
@@ -245,70 +257,54 @@ __global__ __launch_bounds__(256) void k_reset_all(NavData nav, AgentArrays A, S
   if (i >= P.n) return;
   const uint32_t gi = P.base + i;
   begin_reset(nav, A, P, gi);
+  A.flags[gi] = kAgentResetOnly;
   Q.reset_list[i] = gi;
   if (i == 0) Q.counts[kQReset] = P.n;
 }
 
+// One wavefront per agent being reset: both snaps of the new episode, its polar observation and
+// its first geodesic query.
 __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  __shared__ SnapLds lds;
   const uint32_t n = Q.counts[kQReset];
+  const int lane = (int)threadIdx.x;
   uint32_t cands = 0;
-  if (i < n) {
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
     const uint32_t gi = Q.reset_list[i];
     const SceneDev& s = nav.scenes[A.scene[gi]];
     float pos[3], goal[3], rot[4];
     load3(A.pos, gi, pos);
     load3(A.goal, gi, goal);
     for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
-    const NavPt a = snap_point(nav, s, pos[0], pos[1], pos[2], &cands);
-    const NavPt b = snap_point(nav, s, goal[0], goal[1], goal[2], &cands);
-    const float axyz[3] = {a.x, a.y, a.z}, bxyz[3] = {b.x, b.y, b.z};
-    store3(A.nav_xyz, gi, axyz);
-    A.nav_ref[gi] = a.ref;
-    store3(A.goal_xyz, gi, bxyz);
-    A.goal_ref[gi] = b.ref;
-    write_polar(A, gi, pos, rot, goal);
-    GeoQuery q;
-    q.a[0] = a.x; q.a[1] = a.y; q.a[2] = a.z; q.a_ref = a.ref;
-    q.b[0] = b.x; q.b[1] = b.y; q.b[2] = b.z; q.b_ref = b.ref;
-    q.scene = A.scene[gi];
-    q.out = gi;
-    Q.reset_queries[i] = q;
-    if (i == 0) {
-      Q.counts[kQResetGeo] = n;
-      atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
+    const NavPt a = snap_point_wave(nav, s, pos[0], pos[1], pos[2], lds, &cands);
+    const NavPt b = snap_point_wave(nav, s, goal[0], goal[1], goal[2], lds, &cands);
+    if (lane == 0) {
+      const float axyz[3] = {a.x, a.y, a.z}, bxyz[3] = {b.x, b.y, b.z};
+      store3(A.nav_xyz, gi, axyz);
+      A.nav_ref[gi] = a.ref;
+      store3(A.goal_xyz, gi, bxyz);
+      A.goal_ref[gi] = b.ref;
+      write_polar(A, gi, pos, rot, goal);
+      GeoQuery q;
+      q.a[0] = a.x; q.a[1] = a.y; q.a[2] = a.z; q.a_ref = a.ref;
+      q.b[0] = b.x; q.b[1] = b.y; q.b[2] = b.z; q.b_ref = b.ref;
+      q.scene = A.scene[gi];
+      q.out = P.total + gi;
+      Q.queries[atomicAdd(&Q.counts[kQGeo], 1u)] = q;
     }
-    atomicAdd((unsigned long long*)&P.counters[kCntSnapCands], (unsigned long long)cands);
   }
+  if (lane == 0 && blockIdx.x == 0 && n) atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
+  if (lane == 0 && cands) atomicAdd((unsigned long long*)&P.counters[kCntSnapCands], (unsigned long long)cands);
 }
 
-__global__ __launch_bounds__(256) void k_reset_finish(AgentArrays A, StepQueues Q) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= Q.counts[kQReset]) return;
-  const uint32_t gi = Q.reset_list[i];
-  const float d = A.geo[gi];
-  A.cum[gi] = 0;
-  A.init[gi] = d;
-  A.info_prev[gi] = d;
-  A.rew_prev[gi] = d;
-  float pos[3];
-  load3(A.pos, gi, pos);
-  store3(A.prev_pos, gi, pos);
-}
-
-template <int G>
 __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries,
                                                  const uint32_t* __restrict__ count, uint32_t* head, float* out,
                                                  GeoSlot* slots, uint64_t* counters) {
-  constexpr int GPW = 64 / G;
-  __shared__ HeapEntry s_heap[GPW][kHeapLds];
-  __shared__ uint16_t s_first[GPW][kHashSize];
-  GeoGroup<G> g;
-  g.lane = (int)(threadIdx.x % G);
-  g.grp = (int)(threadIdx.x / G);
-  g.heap_lds = s_heap[g.grp];
-  g.first = s_first[g.grp];
-  g.ws = &slots[(size_t)blockIdx.x * GPW + g.grp];
+  __shared__ GeoLds lds;
+  GeoWave g;
+  g.lane = (int)threadIdx.x;
+  g.L = &lds;
+  g.ws = &slots[blockIdx.x];
   g.heapSize = 0;
   g.nodeCount = 0;
   const uint32_t nq = *count;
@@ -316,12 +312,13 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
   for (;;) {
     uint32_t qi = 0;
     if (g.lane == 0) qi = atomicAdd(head, 1u);
-    qi = (uint32_t)__shfl((int)qi, 0, G);
+    qi = (uint32_t)uniform_i((int)qi);
     if (qi >= nq) break;
     const GeoQuery q = queries[qi];
-    const float d = geodesic_query<G>(g, nav, q, &pops, &corridor);
+    const float d = geodesic_query(g, nav, q, &pops, &corridor);
     if (g.lane == 0) out[q.out] = d;
     done++;
+    wave_sync();
   }
   if (g.lane == 0 && done) {
     atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)done);
@@ -331,13 +328,17 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
 }
 
 // ---- batched PathFinder-level kernels (one lane per item, or one group per item)
-__global__ void k_snap_batch(NavData nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref) {
-  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
+__global__ __launch_bounds__(64) void k_snap_batch(NavData nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz,
+                                                   uint32_t* oref) {
+  __shared__ SnapLds lds;
   uint32_t c = 0;
-  const NavPt r = snap_point(nav, nav.scenes[scene], pts[(size_t)i * 3], pts[(size_t)i * 3 + 1], pts[(size_t)i * 3 + 2], &c);
-  oxyz[(size_t)i * 3] = r.x; oxyz[(size_t)i * 3 + 1] = r.y; oxyz[(size_t)i * 3 + 2] = r.z;
-  oref[i] = r.ref;
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
+    const NavPt r = snap_point_wave(nav, nav.scenes[scene], pts[(size_t)i * 3], pts[(size_t)i * 3 + 1], pts[(size_t)i * 3 + 2], lds, &c);
+    if (threadIdx.x == 0) {
+      oxyz[(size_t)i * 3] = r.x; oxyz[(size_t)i * 3 + 1] = r.y; oxyz[(size_t)i * 3 + 2] = r.z;
+      oref[i] = r.ref;
+    }
+  }
 }
 __global__ void k_try_step_batch(NavData nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
                                  uint32_t n, float* oxyz, uint32_t* oref) {
@@ -377,42 +378,38 @@ static inline dim3 grid_for(uint32_t n, uint32_t block) { return dim3((n + block
 
 void launch_geodesic(const NavData& nav, const GeoQuery* queries, const uint32_t* count, uint32_t* head, float* out,
                      GeoSlot* slots, uint32_t num_blocks, uint64_t* counters, hipStream_t st) {
-  // head is cleared by k_clear_queues / k_set_u32 before the producer kernel runs
-  hipLaunchKernelGGL(k_geodesic<kGeoGroup>, dim3(num_blocks), dim3(64), 0, st, nav, queries, count, head, out, slots, counters);
+  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(64), 0, st, nav, queries, count, head, out, slots, counters);
 }
 
 void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
-                 const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, hipStream_t st, hipEvent_t* ev) {
+                 const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st,
+                 hipEvent_t* ev) {
   int e = 0;
   auto mark = [&]() { if (ev) (void)hipEventRecord(ev[e++], st); };
   mark();
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
   hipLaunchKernelGGL(k_step_move, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P, actions_dev);
   mark();
-  launch_geodesic(nav, Q.step_queries, &Q.counts[kQStepGeo], &Q.counts[kQStepGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
   mark();
-  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
+  launch_geodesic(nav, Q.queries, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, slots, geo_blocks, P.counters, st);
   mark();
-  hipLaunchKernelGGL(k_reset_snap, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P);
-  mark();
-  launch_geodesic(nav, Q.reset_queries, &Q.counts[kQResetGeo], &Q.counts[kQResetGeoHead], A.geo, slots, geo_blocks, P.counters, st);
-  mark();
-  hipLaunchKernelGGL(k_reset_finish, grid_for(P.n, 256), dim3(256), 0, st, A, Q);
+  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
   mark();
 }
 
 void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P, GeoSlot* slots,
-                  uint32_t geo_blocks, hipStream_t st) {
+                  uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st) {
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
   hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
-  hipLaunchKernelGGL(k_reset_snap, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P);
-  launch_geodesic(nav, Q.reset_queries, &Q.counts[kQResetGeo], &Q.counts[kQResetGeoHead], A.geo, slots, geo_blocks, P.counters, st);
-  hipLaunchKernelGGL(k_reset_finish, grid_for(P.n, 256), dim3(256), 0, st, A, Q);
+  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
+  launch_geodesic(nav, Q.queries, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
 }
 
 void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref,
-                       hipStream_t st) {
-  hipLaunchKernelGGL(k_snap_batch, grid_for(n, 64), dim3(64), 0, st, nav, scene, pts, n, oxyz, oref);
+                       uint32_t snap_blocks, hipStream_t st) {
+  hipLaunchKernelGGL(k_snap_batch, dim3(snap_blocks < n ? snap_blocks : n), dim3(64), 0, st, nav, scene, pts, n, oxyz, oref);
 }
 void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
                            uint32_t n, float* oxyz, uint32_t* oref, hipStream_t st) {

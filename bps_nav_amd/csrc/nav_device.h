@@ -196,18 +196,142 @@ BPSX_DEV NavPt snap_point(const NavData& nav, const SceneDev& s, float px, float
 #pragma unroll
     for (int k = 0; k < 3; ++k)
       if (box.bmin[k] > nd.bmax[k] || box.bmax[k] < nd.bmin[k]) overlap = false;
-    const bool leaf = nd.i >= 0;
+    const bool leaf = nd.b == kBVLeaf;
     if (leaf && overlap) {
-      const PolyRec& r = nav.polys[s.poly_base + (uint32_t)nd.i];
+      const PolyRec& r = nav.polys[s.poly_base + (uint32_t)nd.a];
       if (r.flags & 1) {
         float cp[3];
         const float d = snap_candidate(nav, s, r, px, py, pz, cp);
         (*ncand)++;
-        if (d < best) { best = d; bestIp = (uint32_t)nd.i; bp[0] = cp[0]; bp[1] = cp[1]; bp[2] = cp[2]; }
+        if (d < best) { best = d; bestIp = (uint32_t)nd.a; bp[0] = cp[0]; bp[1] = cp[1]; bp[2] = cp[2]; }
       }
     }
     if (overlap || leaf) i++;
-    else i += (uint32_t)(-nd.i);
+    else i += (uint32_t)nd.a;
+  }
+  if (bestIp == kInvalidPoly || isnan(bp[0])) return out;
+  out.x = bp[0]; out.y = bp[1]; out.z = bp[2];
+  out.ref = s.ref_base | bestIp;
+  return out;
+}
+
+// snapPoint by a whole wavefront (64 lanes), for callers where few points are snapped at a
+// time.  The BV tree is descended level by level through an LDS frontier (every lane tests
+// one node per round), the leaves that overlap the query box become candidates, each lane
+// evaluates one candidate, and the winner is the smallest (distance, position in the tree's
+// node array): the same polygon the in-order walk with its strict '<' picks.
+constexpr int kSnapFrontier = 1024;
+struct SnapLds {
+  uint16_t frontier[2][kSnapFrontier];
+  uint16_t cand_node[64];   // tree position of the candidates of the current batch
+  uint16_t cand_poly[64];
+};
+BPSX_DEV NavPt snap_point_wave(const NavData& nav, const SceneDev& s, float px, float py, float pz, SnapLds& L,
+                               uint32_t* ncand) {
+  const int lane = (int)(threadIdx.x & 63);
+  const float qnan = __int_as_float(0x7fc00000);
+  NavPt out{qnan, qnan, qnan, 0};
+  if (!finite3(px, py, pz)) return out;
+  const SnapBox box = snap_box(s, px, py, pz);
+  if (!box.hit_tile || s.bv_count == 0) return out;
+  if (!s.bv_tree_ok) return snap_point(nav, s, px, py, pz, ncand);  // every lane walks the same tree
+  float best = 3.402823466e+38f;   // per-lane running best
+  uint32_t bestKey = 0xffffffffu;  // tree position of the lane's best candidate
+  uint32_t bestIp = kInvalidPoly;
+  float bp[3] = {0, 0, 0};
+  int ncands = 0;  // candidates waiting in the batch (uniform)
+  auto flush = [&]() {
+    if (lane < ncands) {
+      const uint32_t ip = L.cand_poly[lane];
+      float cp[3];
+      const float d = snap_candidate(nav, s, nav.polys[s.poly_base + ip], px, py, pz, cp);
+      const uint32_t key = L.cand_node[lane];
+      if (d < best || (d == best && d < 3.402823466e+38f && key < bestKey)) {
+        best = d; bestKey = key; bestIp = ip; bp[0] = cp[0]; bp[1] = cp[1]; bp[2] = cp[2];
+      }
+    }
+    *ncand += (uint32_t)ncands;
+    ncands = 0;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+  // roots: the tree proper and whatever the builder left behind it in the array
+  int nf = 0, cur = 0;
+  {
+    uint32_t k = 0;
+    while (k < s.bv_count && nf < kSnapFrontier) {
+      if (lane == 0) L.frontier[0][nf] = (uint16_t)k;
+      nf++;
+      const BVNodeDev nd = nav.bv[s.bv_base + k];
+      k += nd.b == kBVLeaf ? 1u : (uint32_t)nd.a;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  bool overflow = false;
+  while (nf > 0 && !overflow) {
+    int nnext = 0;
+    for (int basei = 0; basei < nf; basei += 64) {
+      const int fi = basei + lane;
+      bool isCand = false, isInner = false;
+      uint32_t node = 0;
+      BVNodeDev nd{};
+      if (fi < nf) {
+        node = L.frontier[cur][fi];
+        nd = nav.bv[s.bv_base + node];
+        bool overlap = true;
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+          if (box.bmin[k] > nd.bmax[k] || box.bmax[k] < nd.bmin[k]) overlap = false;
+        if (overlap) {
+          if (nd.b == kBVLeaf) isCand = (nav.polys[s.poly_base + nd.a].flags & 1) != 0;
+          else isInner = true;
+        }
+      }
+      // children of overlapping inner nodes go to the next frontier
+      const unsigned long long mi = __ballot(isInner);
+      const int ni = __popcll(mi);
+      if (nnext + 2 * ni > kSnapFrontier) { overflow = true; break; }
+      if (isInner) {
+        const int pos = nnext + 2 * __popcll(mi & ((1ull << lane) - 1ull));
+        L.frontier[cur ^ 1][pos] = (uint16_t)(node + 1);
+        L.frontier[cur ^ 1][pos + 1] = nd.b;
+      }
+      nnext += 2 * ni;
+      // overlapping walkable leaves join the candidate batch; a full batch is evaluated
+      unsigned long long mc = __ballot(isCand);
+      while (mc) {
+        const int room = 64 - ncands;
+        const int take = min(room, (int)__popcll(mc));
+        const int rank = __popcll(mc & ((1ull << lane) - 1ull));
+        if (isCand && rank < take) {
+          L.cand_node[ncands + rank] = (uint16_t)node;
+          L.cand_poly[ncands + rank] = nd.a;
+          isCand = false;
+        }
+        ncands += take;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (ncands == 64) flush();
+        mc = __ballot(isCand);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    cur ^= 1;
+    nf = nnext;
+  }
+  if (overflow) return snap_point(nav, s, px, py, pz, ncand);
+  if (ncands) flush();
+  // wave-wide minimum of (distance, tree position)
+  for (int o = 32; o > 0; o >>= 1) {
+    const float od = __shfl_xor(best, o);
+    const uint32_t ok = (uint32_t)__shfl_xor((int)bestKey, o);
+    const uint32_t oi = (uint32_t)__shfl_xor((int)bestIp, o);
+    const float o0 = __shfl_xor(bp[0], o), o1 = __shfl_xor(bp[1], o), o2 = __shfl_xor(bp[2], o);
+    const bool mineValid = bestIp != kInvalidPoly, otherValid = oi != kInvalidPoly;
+    const bool takeOther = otherValid && (!mineValid || od < best || (od == best && ok < bestKey));
+    if (takeOther) { best = od; bestKey = ok; bestIp = oi; bp[0] = o0; bp[1] = o1; bp[2] = o2; }
   }
   if (bestIp == kInvalidPoly || isnan(bp[0])) return out;
   out.x = bp[0]; out.y = bp[1]; out.z = bp[2];

@@ -184,13 +184,46 @@ int parse_navmesh(const uint8_t* b, size_t n, HostScene* out) {
     r.area_cum = acc;
   }
 
-  // BV tree: leaves must name valid polygons, escapes must move forward
+  // BV tree: repack dtBVNode (bounds + int) into BVNodeDev.  Leaves must name valid polygons;
+  // an internal node at i with escape e owns nodes (i, i+e): its left child is i+1 and its
+  // right child follows the left subtree.  The links are verified so that the kernels'
+  // descent always moves to larger indices inside the array.
   s.bv.assign((size_t)h.bvNodeCount, BVNodeDev{});
-  if (h.bvNodeCount) memcpy(s.bv.data(), bvp, (size_t)h.bvNodeCount * sizeof(BVNodeDev));
-  for (int i = 0; i < h.bvNodeCount; ++i) {
-    const int32_t v = s.bv[i].i;
-    if (v >= np) return fail(BPSX_E_INVAL, "navmesh: BV leaf out of range");
-    if (v < 0 && -(int64_t)v < 1) return fail(BPSX_E_INVAL, "navmesh: BV escape index must be positive");
+  bool tree_ok = h.bvNodeCount > 0;
+  {
+    std::vector<TileBVNode> raw((size_t)h.bvNodeCount);
+    if (h.bvNodeCount) memcpy(raw.data(), bvp, (size_t)h.bvNodeCount * sizeof(TileBVNode));
+    const int64_t cnt = h.bvNodeCount;
+    auto size_of = [&](int64_t i) -> int64_t { return raw[(size_t)i].i >= 0 ? 1 : -(int64_t)raw[(size_t)i].i; };
+    for (int64_t i = 0; i < cnt; ++i) {
+      const TileBVNode& r = raw[(size_t)i];
+      BVNodeDev& o = s.bv[(size_t)i];
+      memcpy(o.bmin, r.bmin, 6);
+      memcpy(o.bmax, r.bmax, 6);
+      if (r.i >= 0) {
+        if (r.i >= np) return fail(BPSX_E_INVAL, "navmesh: BV leaf out of range");
+        o.a = (uint16_t)r.i;
+        o.b = kBVLeaf;
+      } else {
+        const int64_t e = -(int64_t)r.i;
+        if (e < 1 || e > 0xfffe) return fail(BPSX_E_INVAL, "navmesh: BV escape offset out of range");
+        o.a = (uint16_t)e;
+        const int64_t left = i + 1;
+        const int64_t right = left < cnt ? left + size_of(left) : cnt;
+        if (left >= cnt || right >= cnt || right >= i + e || right + size_of(right) != i + e) {
+          tree_ok = false;
+          o.b = (uint16_t)(left < cnt ? left : 0);
+        } else {
+          o.b = (uint16_t)right;
+        }
+      }
+    }
+    // the builder reserves 2N nodes and uses 2N-1: the rest are zero leaves outside the tree;
+    // the in-order walk visits them, so the descent must too (they are appended to its frontier)
+    if (tree_ok) {
+      const int64_t root_size = size_of(0);
+      if (root_size > cnt) tree_ok = false;
+    }
   }
 
   SceneDev& d = s.dev;
@@ -208,6 +241,7 @@ int parse_navmesh(const uint8_t* b, size_t n, HostScene* out) {
   d.qfac = h.bvQuantFactor;
   d.climb = h.walkableClimb;
   d.area_total = acc;
+  d.bv_tree_ok = tree_ok ? 1u : 0u;
   return BPSX_OK;
 }
 

@@ -121,7 +121,7 @@ int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
  * elapsed times up.  get_kernel_times returns the sums in milliseconds and the number of
  * steps they cover; enabling clears the sums. */
-#define BPSX_NUM_KERNELS 6
+#define BPSX_NUM_KERNELS 4
 int bpsx_set_profiling(bpsx_sim *sim, int enabled);
 int bpsx_get_kernel_times(bpsx_sim *sim, double *out_ms_sum /* [BPSX_NUM_KERNELS] */,
                           uint64_t *out_steps);
