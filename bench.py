@@ -23,6 +23,9 @@ HBM_PEAK_GBS = 8000.0
 # end polygons are read once more for the boundary clamp, 2 * (32 + 12 * nv) with nv = 4.
 BYTES_PER_CORRIDOR_POLY = 60
 BYTES_PER_QUERY_ENDS = 2 * (32 + 12 * 4)
+# HBM bytes per k_geodesic launch at the default workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file scaled by a 256 MiB copy (profiles/k_geodesic_c4_hbm_traffic.md).
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 1.126e9
 
 
 def log(*a):
@@ -94,6 +97,9 @@ def main():
     ap.add_argument("--agents", type=int, default=16384)
     ap.add_argument("--scenes", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy, so a counter profile of this command holds a "
+                         "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1 (agents are independent, so a "
@@ -115,6 +121,12 @@ def main():
     p_turn = (1.0 - p_forward - 0.04) / 2
     probs = torch.tensor([0.04, p_forward, p_turn, p_turn])
     actions = torch.multinomial(probs.expand(K + W, 4), N, replacement=True, generator=g).to(torch.int64).cuda()
+    if args.calib_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     gen.reset(0)
     for t in range(W):
         gen.step(0, actions[t])
@@ -143,7 +155,9 @@ def main():
     geo_ms = kt["geodesic"]
     achieved = geo_bytes / K / (geo_ms * 1e-3) / 1e9 if geo_ms > 0 else 0.0
     roofline = {"bound": "hbm", "kernel": "k_geodesic", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None, "dominant_kernel_by_time": dominant,
+                "frac": achieved / HBM_PEAK_GBS,
+                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (N, S) == (16384, 128) else None,
+                "dominant_kernel_by_time": dominant,
                 "kernel_ms_per_step": kt, "algorithmic_bytes_per_step": geo_bytes / K}
     gen.close()
     result = {

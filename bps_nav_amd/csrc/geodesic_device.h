@@ -21,7 +21,7 @@
 namespace bpsx {
 
 constexpr int kNodesLds = 512;   // nodes kept in LDS per query
-constexpr int kHeapLds = 512;    // open-list entries kept in LDS per query
+constexpr int kHeapLds = 384;    // open-list entries kept in LDS per query
 constexpr int kHashSize = 512;
 
 BPSX_DEV void wave_sync() {
@@ -42,8 +42,7 @@ struct GeoLds {
   uint32_t n_meta[kNodesLds];      // id:15 | flags:2 << 15 | pidx:12 << 17
   uint16_t n_next[kNodesLds];
   uint16_t first[kHashSize];
-  float h_total[kHeapLds];
-  uint16_t h_node[kHeapLds];
+  HeapEntry heap[kHeapLds];
 };
 // After A* the node arrays are dead; the funnel reuses them for the corridor and its portals.
 struct FunnelLds {
@@ -131,11 +130,13 @@ struct GeoWave {
   }
 
   // ---------------------------------------------------------------- open list
-  BPSX_DEV float ht(int i) const { return i < kHeapLds ? L->h_total[i] : ws->heap_spill[i].total; }
-  BPSX_DEV int hn(int i) const { return i < kHeapLds ? (int)L->h_node[i] : (int)ws->heap_spill[i].node; }
+  BPSX_DEV HeapEntry hget(int i) const { return i < kHeapLds ? L->heap[i] : ws->heap_spill[i]; }
+  BPSX_DEV float ht(int i) const { return hget(i).total; }
+  BPSX_DEV int hn(int i) const { return (int)hget(i).node; }
   BPSX_DEV void hset(int i, float t, int n) const {
-    if (i < kHeapLds) { L->h_total[i] = t; L->h_node[i] = (uint16_t)n; }
-    else { ws->heap_spill[i].total = t; ws->heap_spill[i].node = (uint32_t)n; }
+    const HeapEntry e{t, (uint32_t)n};
+    if (i < kHeapLds) L->heap[i] = e;
+    else ws->heap_spill[i] = e;
   }
   // dtNodeQueue::bubbleUp from index i0 with entry (t, n), all ancestors looked at at once:
   // along a leaf-to-root path the keys never increase, so the ancestors that are greater than
@@ -146,7 +147,7 @@ struct GeoWave {
     const bool valid = lane >= 1 && a >= 0;
     float at = 0;
     int an = 0;
-    if (valid) { at = ht(a); an = hn(a); }
+    if (valid) { const HeapEntry e = hget(a); at = e.total; an = (int)e.node; }
     const unsigned long long gt = __ballot(valid && at > t);
     const int m = __popcll(gt);  // ancestors 1..m move down
     wave_sync();
@@ -180,8 +181,9 @@ struct GeoWave {
     heapSize--;
     const int size = heapSize;
     if (size == 0) return top;
-    const float lt = ht(size);
-    const int ln = hn(size);
+    const HeapEntry lastE = hget(size);
+    const float lt = lastE.total;
+    const int ln = (int)lastE.node;
     // route entries are collected one per lane: lane d keeps the d-th node of the route
     float myT = 0;
     int myN = 0, myIdx = -1, myParent = -1;
@@ -197,11 +199,12 @@ struct GeoWave {
       int cn = 0;
       if (lane < 63) {
         const int c1 = 2 * node + 1;
-        if (c1 < size && node < size) {
-          ct = ht(c1); cn = hn(c1); choice = c1;
+        if (c1 < size) {
+          const HeapEntry e1 = hget(c1);
+          ct = e1.total; cn = (int)e1.node; choice = c1;
           if (c1 + 1 < size) {
-            const float t2 = ht(c1 + 1);
-            if (ct > t2) { ct = t2; cn = hn(c1 + 1); choice = c1 + 1; }
+            const HeapEntry e2 = hget(c1 + 1);
+            if (ct > e2.total) { ct = e2.total; cn = (int)e2.node; choice = c1 + 1; }
           }
         }
       }
@@ -274,6 +277,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       nbRaw = bp->nei[lane];
       nbWalk = bp->walk[lane];
       l0 = bp->v[lane][0]; l1 = bp->v[lane][1]; l2 = bp->v[lane][2];
+      if (lane + 1 < kNvp) { r0 = bp->v[lane + 1][0]; r1 = bp->v[lane + 1][1]; r2 = bp->v[lane + 1][2]; }
     }
     const uint32_t pidx = meta_pidx(best.meta);
     const uint32_t parentIp = pidx ? meta_id(g.node_meta((int)pidx - 1)) : kInvalidPoly;
@@ -282,10 +286,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     wave_sync();
     if (bestIp == endIp) { lastBest = bi; break; }
     (*pops)++;
-    // right end of edge j is the left end of edge j+1 (mod nv)
+    // right end of edge j is vertex j+1, wrapping to vertex 0 on the last edge
     {
-      const int nxt = lane + 1 < nv ? lane + 1 : 0;
-      r0 = __shfl(l0, nxt); r1 = __shfl(l1, nxt); r2 = __shfl(l2, nxt);
+      const float w0 = lane_f(l0, 0), w1 = lane_f(l1, 0), w2 = lane_f(l2, 0);
+      if (lane + 1 >= nv) { r0 = w0; r1 = w1; r2 = w2; }
     }
     // ---- per-edge phase: lane j looks at edge j
     uint32_t nb = kInvalidPoly;
@@ -295,10 +299,13 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     }
     // a polygon reached through two edges of the same expansion: the second visit never
     // changes the node (same position, same cost), so only the first edge counts
+    {
+      const uint32_t orig = nb;
 #pragma unroll
-    for (int k = 0; k < kNvp - 1; ++k) {
-      const uint32_t other = (uint32_t)__shfl((int)nb, k);
-      if (lane > k && nb != kInvalidPoly && other == nb) nb = kInvalidPoly;
+      for (int k = 0; k < kNvp - 1; ++k) {
+        const uint32_t other = (uint32_t)lane_i((int)orig, k);
+        if (lane > k && other == orig) nb = kInvalidPoly;
+      }
     }
     int ni = -1;
     if (nb != kInvalidPoly) ni = g.find(nb);
