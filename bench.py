@@ -143,7 +143,10 @@ def main():
     gen.check_errors()
     c1 = gen.counters()
     kt, profiled = gen.kernel_times()
-    d = {k: c1[k] - c0[k] for k in c1}
+    d = {k: c1[k] - c0[k] for k in c1 if k != "phase_cycles"}
+    if any(c1["phase_cycles"]):
+        ph = [a - b for a, b in zip(c1["phase_cycles"], c0["phase_cycles"])]
+        log("A* phase cycles per expanded node (diagnostic build): " + " ".join(f"{v / max(1, d['astar_pops']):.0f}" for v in ph))
     dist = gen.get_infos(0)["distanceToGoal"].cpu().numpy()
     log(f"timed {K} steps in {elapsed:.3f}s; per-kernel ms/step {json.dumps({k: round(v, 4) for k, v in kt.items()})}")
     log(f"per step: {d['geodesic_queries'] / K:.0f} geodesic queries, {d['astar_pops'] / max(1, d['geodesic_queries']):.0f} "

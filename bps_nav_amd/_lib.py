@@ -7,7 +7,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libbpsx.so")
+LIB_PATH = os.environ.get("BPSX_LIBRARY") or os.path.join(_HERE, "libbpsx.so")
 
 
 class Config(C.Structure):

@@ -202,11 +202,13 @@ class PointNavRolloutGenerator:
         _lib.check(self._L.bpsx_check_errors(self._h))
 
     def counters(self):
-        out = np.zeros(8, np.uint64)
+        out = np.zeros(16, np.uint64)
         _lib.check(self._L.bpsx_get_counters(self._h, out.ctypes.data))
         names = ["agent_steps", "forward_moves", "geodesic_queries", "astar_pops", "corridor_polys", "resets",
                  "move_polys", "snap_candidates"]
-        return dict(zip(names, (int(v) for v in out)))
+        d = dict(zip(names, (int(v) for v in out[:8])))
+        d["phase_cycles"] = [int(v) for v in out[8:]]
+        return d
 
     def set_profiling(self, enabled):
         _lib.check(self._L.bpsx_set_profiling(self._h, int(enabled)))

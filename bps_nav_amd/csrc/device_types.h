@@ -83,6 +83,7 @@ struct AgentArrays {
   uint32_t* episode;  // [N]
   uint32_t* nresets;  // [N]
   uint32_t* flags;    // [N] transient per-step bits, see kAgent*
+  uint32_t* dist_ok;  // [N] 1 when info_prev is the goal->agent distance of the current navmesh point
   float* geo;         // [2N] geodesic results: [i] step query of agent i, [N + i] its reset query
   // outputs
   float* rewards;     // [N]
@@ -90,7 +91,7 @@ struct AgentArrays {
   float* infos;       // [N][3]
   float* polars;      // [N][2]
 };
-constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentSkip = 8u, kAgentResetOnly = 16u;
+constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentReuse = 4u, kAgentSkip = 8u, kAgentResetOnly = 16u;
 
 struct NavData {
   const PolyRec* polys;

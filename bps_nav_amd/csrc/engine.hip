@@ -190,7 +190,7 @@ int bpsx_finalize(bpsx_sim* sim) {
       (rc = sim->alloc(&A.goal_ref, N)) || (rc = sim->alloc(&A.prev_pos, N * 3)) || (rc = sim->alloc(&A.info_prev, N)) ||
       (rc = sim->alloc(&A.cum, N)) || (rc = sim->alloc(&A.init, N)) || (rc = sim->alloc(&A.rew_prev, N)) ||
       (rc = sim->alloc(&A.step, N)) || (rc = sim->alloc(&A.scene, N)) || (rc = sim->alloc(&A.episode, N)) ||
-      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.geo, 2 * N)) ||
+      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.dist_ok, N)) || (rc = sim->alloc(&A.geo, 2 * N)) ||
       (rc = sim->alloc(&A.rewards, N)) || (rc = sim->alloc(&A.masks, N)) || (rc = sim->alloc(&A.infos, N * 3)) ||
       (rc = sim->alloc(&A.polars, N * 2)))
     return rc;

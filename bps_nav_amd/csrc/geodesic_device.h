@@ -20,6 +20,12 @@
 
 namespace bpsx {
 
+#ifdef BPSX_PHASE_TIMING
+#define PHASE_MARK(k) do { const unsigned long long now_ = __builtin_readcyclecounter(); phase_acc[k] += now_ - phase_t0; phase_t0 = now_; } while (0)
+#else
+#define PHASE_MARK(k) do { } while (0)
+#endif
+
 constexpr int kNodesLds = 512;   // nodes kept in LDS per query
 constexpr int kHeapLds = 384;    // open-list entries kept in LDS per query
 constexpr int kHashSize = 512;
@@ -238,8 +244,15 @@ struct GeoWave {
 // Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
 // when the reference would report anything but plain DT_SUCCESS.
 BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev& s, uint32_t startIp, uint32_t endIp,
-                   const float* startPos, const float* endPos, uint32_t* pops) {
+                   const float* startPos, const float* endPos, uint32_t* pops
+#ifdef BPSX_PHASE_TIMING
+                   , unsigned long long* phase_acc
+#endif
+                   ) {
   const int lane = g.lane;
+#ifdef BPSX_PHASE_TIMING
+  unsigned long long phase_t0 = __builtin_readcyclecounter();
+#endif
   if (startIp == endIp) {
     if (lane == 0) F->corridor[0] = (uint16_t)startIp;
     wave_sync();
@@ -281,7 +294,9 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     }
     const uint32_t pidx = meta_pidx(best.meta);
     const uint32_t parentIp = pidx ? meta_id(g.node_meta((int)pidx - 1)) : kInvalidPoly;
+    PHASE_MARK(0);
     g.pop();
+    PHASE_MARK(1);
     if (lane == 0) g.node_set_meta(bi, meta_pack(bestIp, (meta_flags(best.meta) & ~1u) | 2u, pidx));
     wave_sync();
     if (bestIp == endIp) { lastBest = bi; break; }
@@ -307,8 +322,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         if (lane > k && other == orig) nb = kInvalidPoly;
       }
     }
+    PHASE_MARK(2);
     int ni = -1;
     if (nb != kInvalidPoly) ni = g.find(nb);
+    PHASE_MARK(3);
     // new nodes take consecutive indices in edge order; past the pool's end they are dropped
     {
       const unsigned long long need = __ballot(nb != kInvalidPoly && ni < 0);
@@ -338,6 +355,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         }
       }
     }
+    PHASE_MARK(4);
     bool update = false;
     float total = 0, heuristic = 0;
     bool wasOpen = false;
@@ -373,6 +391,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       }
     }
     wave_sync();
+    PHASE_MARK(5);
     // ---- ordered phase: heap and "nearest so far" updates in edge order
     unsigned long long upd = __ballot(update);
     while (upd) {
@@ -386,6 +405,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       else g.push(t, node);
       if (h < lastBestCost) { lastBestCost = h; lastBest = node; }
     }
+    PHASE_MARK(6);
   }
   // getPathToNode
   int length = 0;
@@ -514,7 +534,11 @@ BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const S
 }
 
 // Full PathFinder::findPath distance for one query, executed by a wavefront.
-BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q, uint32_t* pops, uint32_t* corridor) {
+BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q, uint32_t* pops, uint32_t* corridor
+#ifdef BPSX_PHASE_TIMING
+                              , unsigned long long* phase_acc
+#endif
+                              ) {
   const float INF = __int_as_float(0x7f800000);
   {
     // Eigen isApprox with default precision; sums of three reduce as a0 + (a1 + a2)
@@ -532,10 +556,17 @@ BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q,
   if (nav.polys[s.poly_base + sIp].island != nav.polys[s.poly_base + eIp].island) return INF;
   if (!finite3(q.a[0], q.a[1], q.a[2]) || !finite3(q.b[0], q.b[1], q.b[2])) return INF;
   FunnelLds* F = reinterpret_cast<FunnelLds*>(g.L);
+#ifdef BPSX_PHASE_TIMING
+  const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops, phase_acc);
+  unsigned long long phase_t0 = __builtin_readcyclecounter();
+#else
   const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops);
+#endif
   if (n <= 0) return INF;
   *corridor += (uint32_t)n;
-  return funnel_length(g.lane, F, nav, s, n, q.a, q.b);
+  const float len = funnel_length(g.lane, F, nav, s, n, q.a, q.b);
+  PHASE_MARK(7);
+  return len;
 }
 
 }  // namespace bpsx

@@ -140,6 +140,10 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
       A.step[gi] = step;
       bool done = (float)step >= P.max_steps;
       bool moved = false;
+      // The goal->agent distance is a deterministic function of the two navmesh points. When
+      // the agent's point is bit-identical to the one the last step query of this episode was
+      // made for (blocked forward move, turn, stop), that query's result is the answer again.
+      bool samePoint = true;
       if (action == 0) {
         done = true;
       } else {
@@ -156,6 +160,8 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
           st.x = A.nav_xyz[(size_t)gi * 3]; st.y = A.nav_xyz[(size_t)gi * 3 + 1]; st.z = A.nav_xyz[(size_t)gi * 3 + 2];
           st.ref = A.nav_ref[gi];
           const NavPt r = try_step(nav, s, st, pos[0] + delta[0], pos[1] + delta[1], pos[2] + delta[2], &movePolys);
+          samePoint = __float_as_uint(r.x) == __float_as_uint(st.x) && __float_as_uint(r.y) == __float_as_uint(st.y) &&
+                      __float_as_uint(r.z) == __float_as_uint(st.z) && r.ref == st.ref;
           pos[0] = r.x; pos[1] = r.y; pos[2] = r.z;
           store3(A.nav_xyz, gi, pos);
           A.nav_ref[gi] = r.ref;
@@ -167,8 +173,9 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         }
         write_polar(A, gi, pos, rot, goal);
       }
-      A.flags[gi] = (done ? kAgentDone : 0u) | (moved ? kAgentMoved : 0u);
-      if (done || moved) {
+      const bool reuse = (done || moved) && samePoint && A.dist_ok[gi] != 0;
+      A.flags[gi] = (done ? kAgentDone : 0u) | (moved ? kAgentMoved : 0u) | (reuse ? kAgentReuse : 0u);
+      if ((done || moved) && !reuse) {
         want = true;
         load3(A.goal_xyz, gi, q.a);
         q.a_ref = A.goal_ref[gi];
@@ -211,14 +218,16 @@ __global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P
   const bool done = f & kAgentDone, moved = f & kAgentMoved;
   if (!(f & kAgentResetOnly)) {
     float dist, success = 0, spl = 0;
+    const float fresh = (f & kAgentReuse) ? A.info_prev[gi] : A.geo[gi];
     if (done) {
-      dist = A.geo[gi];
+      dist = fresh;
       success = dist < 0.2f ? 1.0f : 0.0f;
       const float init = A.init[gi], cum = A.cum[gi];
       const float mx = init < cum ? cum : init;
       spl = success * init / mx;
     } else if (moved) {
-      dist = A.geo[gi];
+      dist = fresh;
+      A.dist_ok[gi] = 1;
       float pos[3], pp[3];
       load3(A.pos, gi, pos);
       load3(A.prev_pos, gi, pp);
@@ -244,7 +253,8 @@ __global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P
     const float d = A.geo[(size_t)P.total + gi];
     A.cum[gi] = 0;
     A.init[gi] = d;
-    A.info_prev[gi] = d;
+    A.info_prev[gi] = d;   // agent->goal: not a goal->agent result, so not reusable
+    A.dist_ok[gi] = 0;
     A.rew_prev[gi] = d;
     float pos[3];
     load3(A.pos, gi, pos);
@@ -309,13 +319,20 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
   g.nodeCount = 0;
   const uint32_t nq = *count;
   uint32_t pops = 0, corridor = 0, done = 0;
+#ifdef BPSX_PHASE_TIMING
+  unsigned long long phase_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
   for (;;) {
     uint32_t qi = 0;
     if (g.lane == 0) qi = atomicAdd(head, 1u);
     qi = (uint32_t)uniform_i((int)qi);
     if (qi >= nq) break;
     const GeoQuery q = queries[qi];
+#ifdef BPSX_PHASE_TIMING
+    const float d = geodesic_query(g, nav, q, &pops, &corridor, phase_acc);
+#else
     const float d = geodesic_query(g, nav, q, &pops, &corridor);
+#endif
     if (g.lane == 0) out[q.out] = d;
     done++;
     wave_sync();
@@ -324,6 +341,9 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
     atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)done);
     atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)pops);
     atomicAdd((unsigned long long*)&counters[kCntCorridor], (unsigned long long)corridor);
+#ifdef BPSX_PHASE_TIMING
+    for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], phase_acc[k]);
+#endif
   }
 }
 
