@@ -44,7 +44,8 @@ class SceneParams(C.Structure):
                 ("door_width", C.c_float), ("clutter_frac", C.c_float), ("maze_w", C.c_uint32),
                 ("maze_h", C.c_uint32), ("corridor_min", C.c_float), ("corridor_max", C.c_float),
                 ("wall", C.c_float), ("braid", C.c_float), ("tri_frac", C.c_float),
-                ("hex_frac", C.c_float), ("origin", C.c_float * 3)]
+                ("hex_frac", C.c_float), ("origin", C.c_float * 3), ("tiles_x", C.c_uint32),
+                ("tiles_z", C.c_uint32)]
 
 
 _lib = None

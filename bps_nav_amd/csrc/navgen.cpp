@@ -422,129 +422,141 @@ void gen_maze(const bpsx_scene_params& p, Grid& g, Rng& rng) {
     }
 }
 
-// Turns the walkable cells into convex polygons (squares, triangle pairs, 2x1 hexagons
-// with collinear mid-edge vertices) with shared-edge adjacency, then packs one tile.
+// Turns the walkable cells into convex polygons (squares, triangle pairs, 2x1 hexagons with
+// collinear mid-edge vertices) with shared-edge adjacency and packs them as tiles_x * tiles_z
+// tiles; polygon edges on a tile border that face a walkable cell become portals.
 int grid_to_mset(const Grid& g, const bpsx_scene_params& p, Rng& rng, std::vector<uint8_t>& mset) {
   const int nx = g.nx, nz = g.nz, cell = (int)p.cell;
-  if ((long)nx * cell > 65000 || (long)nz * cell > 65000) return fail(BPSX_E_INVAL, "gen_scene: grid too large for 16-bit vertices");
+  const int ntx = std::max(1, (int)p.tiles_x), ntz = std::max(1, (int)p.tiles_z);
+  const int tw = (nx + ntx - 1) / ntx, th = (nz + ntz - 1) / ntz;  // tile size in cells
+  if ((long)tw * cell > 65000 || (long)th * cell > 65000) return fail(BPSX_E_INVAL, "gen_scene: tile too large for 16-bit vertices");
+  std::vector<std::vector<uint8_t>> tiles;
+  uint32_t maxPolys = 0;
   // cell sides: 0 = x- (west), 1 = z+ , 2 = x+ (east), 3 = z-
   std::vector<int32_t> sidePoly((size_t)nx * nz * 4, -1);
-  std::vector<int8_t> sideEdge((size_t)nx * nz * 4, -1);
-  std::vector<int32_t> vmap((size_t)(nx + 1) * (nz + 1), -1);
-  std::vector<uint16_t> verts;
-  struct P { int nv; int32_t v[6]; int32_t nei[6]; int cx[6], cz[6], side[6]; };
-  std::vector<P> polys;
   std::vector<uint8_t> used((size_t)nx * nz, 0);
-  auto vid = [&](int ix, int iz) {
-    int32_t& m = vmap[(size_t)iz * (nx + 1) + ix];
-    if (m < 0) {
-      m = (int32_t)(verts.size() / 3);
-      verts.push_back((uint16_t)(ix * cell));
-      verts.push_back(0);
-      verts.push_back((uint16_t)(iz * cell));
-    }
-    return m;
-  };
-  auto own = [&](int x, int z, int side, int poly, int edge) {
-    sidePoly[((size_t)z * nx + x) * 4 + side] = poly;
-    sideEdge[((size_t)z * nx + x) * 4 + side] = (int8_t)edge;
-  };
-  for (int z = 0; z < nz; ++z)
-    for (int x = 0; x < nx; ++x) {
-      if (!g.get(x, z) || used[(size_t)z * nx + x]) continue;
-      used[(size_t)z * nx + x] = 1;
-      const double r = rng.uni();
-      if (r < p.hex_frac && g.get(x + 1, z) && !used[(size_t)z * nx + x + 1]) {
-        used[(size_t)z * nx + x + 1] = 1;
-        // (x1,z0),(x0,z0),(x0,z1),(x1,z1),(x2,z1),(x2,z0): every fan triangle from
-        // vertex 0 has positive area.
-        P q{}; q.nv = 6;
-        const int id = (int)polys.size();
-        q.v[0] = vid(x + 1, z);     q.v[1] = vid(x, z);         q.v[2] = vid(x, z + 1);
-        q.v[3] = vid(x + 1, z + 1); q.v[4] = vid(x + 2, z + 1); q.v[5] = vid(x + 2, z);
-        for (int e = 0; e < 6; ++e) q.nei[e] = -1;
-        // e0: (x1,z0)->(x0,z0) = cell x side z-; e1: west of cell x; e2: z+ of cell x;
-        // e3: z+ of cell x+1; e4: east of cell x+1; e5: z- of cell x+1
-        const int ecx[6] = {x, x, x, x + 1, x + 1, x + 1};
-        const int esd[6] = {3, 0, 1, 1, 2, 3};
-        for (int e = 0; e < 6; ++e) { q.cx[e] = ecx[e]; q.cz[e] = z; q.side[e] = esd[e]; own(ecx[e], z, esd[e], id, e); }
-        polys.push_back(q);
-      } else if (r < p.hex_frac + p.tri_frac) {
-        const int id = (int)polys.size();
-        P a{}, b{}; a.nv = b.nv = 3;
-        for (int e = 0; e < 6; ++e) { a.nei[e] = b.nei[e] = -1; a.side[e] = b.side[e] = -1; }
-        if (rng.next() & 1) {
-          // diagonal (x0,z0)-(x1,z1)
-          a.v[0] = vid(x, z); a.v[1] = vid(x, z + 1); a.v[2] = vid(x + 1, z + 1);
-          a.side[0] = 0; a.side[1] = 1; a.nei[2] = id + 1;
-          b.v[0] = vid(x, z); b.v[1] = vid(x + 1, z + 1); b.v[2] = vid(x + 1, z);
-          b.nei[0] = id; b.side[1] = 2; b.side[2] = 3;
-        } else {
-          // diagonal (x0,z1)-(x1,z0)
-          a.v[0] = vid(x, z); a.v[1] = vid(x, z + 1); a.v[2] = vid(x + 1, z);
-          a.side[0] = 0; a.nei[1] = id + 1; a.side[2] = 3;
-          b.v[0] = vid(x, z + 1); b.v[1] = vid(x + 1, z + 1); b.v[2] = vid(x + 1, z);
-          b.side[0] = 1; b.side[1] = 2; b.nei[2] = id;
-        }
-        for (int e = 0; e < 3; ++e) {
-          a.cx[e] = b.cx[e] = x; a.cz[e] = b.cz[e] = z;
-          if (a.side[e] >= 0) own(x, z, a.side[e], id, e);
-          if (b.side[e] >= 0) own(x, z, b.side[e], id + 1, e);
-        }
-        polys.push_back(a);
-        polys.push_back(b);
-      } else {
-        P q{}; q.nv = 4;
-        const int id = (int)polys.size();
-        q.v[0] = vid(x, z); q.v[1] = vid(x, z + 1); q.v[2] = vid(x + 1, z + 1); q.v[3] = vid(x + 1, z);
-        for (int e = 0; e < 4; ++e) { q.nei[e] = -1; q.cx[e] = x; q.cz[e] = z; q.side[e] = e; own(x, z, e, id, e); }
-        polys.push_back(q);
-      }
-    }
-  if (polys.empty()) return fail(BPSX_E_INVAL, "gen_scene: no walkable cells");
-  if (polys.size() > 0x7fff) return fail(BPSX_E_INVAL, "gen_scene: more than 32767 polygons; reduce the layout or enlarge the cell");
-  if (verts.size() / 3 >= 0xffff) return fail(BPSX_E_INVAL, "gen_scene: too many vertices");
   const int odx[4] = {-1, 0, 1, 0}, odz[4] = {0, 1, 0, -1};
-  const int np = (int)polys.size();
-  std::vector<uint16_t> pk((size_t)np * 12, 0xffff);
-  std::vector<uint16_t> flags((size_t)np, kPolyFlagWalk);
-  std::vector<uint8_t> areas((size_t)np, 0);
-  for (int i = 0; i < np; ++i) {
-    P& q = polys[i];
-    for (int e = 0; e < q.nv; ++e) {
-      pk[(size_t)i * 12 + e] = (uint16_t)q.v[e];
-      int nei = q.nei[e];
-      if (nei < 0 && q.side[e] >= 0) {
-        const int ax = q.cx[e] + odx[q.side[e]], az = q.cz[e] + odz[q.side[e]];
-        if (g.in(ax, az) && g.get(ax, az)) nei = sidePoly[((size_t)az * nx + ax) * 4 + ((q.side[e] + 2) & 3)];
+  for (int tz = 0; tz < ntz; ++tz)
+    for (int tx = 0; tx < ntx; ++tx) {
+      const int x0 = tx * tw, x1 = std::min(nx, x0 + tw), z0 = tz * th, z1 = std::min(nz, z0 + th);
+      std::vector<int32_t> vmap((size_t)(tw + 1) * (th + 1), -1);
+      std::vector<uint16_t> verts;
+      struct P { int nv; int32_t v[6]; int32_t nei[6]; int cx[6], cz[6], side[6]; };
+      std::vector<P> polys;
+      auto vid = [&](int ix, int iz) {
+        int32_t& m = vmap[(size_t)(iz - z0) * (tw + 1) + (ix - x0)];
+        if (m < 0) {
+          m = (int32_t)(verts.size() / 3);
+          verts.push_back((uint16_t)((ix - x0) * cell));
+          verts.push_back(0);
+          verts.push_back((uint16_t)((iz - z0) * cell));
+        }
+        return m;
+      };
+      auto own = [&](int x, int z, int side, int poly) { sidePoly[((size_t)z * nx + x) * 4 + side] = poly; };
+      for (int z = z0; z < z1; ++z)
+        for (int x = x0; x < x1; ++x) {
+          if (!g.get(x, z) || used[(size_t)z * nx + x]) continue;
+          used[(size_t)z * nx + x] = 1;
+          const double r = rng.uni();
+          if (r < p.hex_frac && x + 1 < x1 && g.get(x + 1, z) && !used[(size_t)z * nx + x + 1]) {
+            used[(size_t)z * nx + x + 1] = 1;
+            // (x1,z0),(x0,z0),(x0,z1),(x1,z1),(x2,z1),(x2,z0): every fan triangle from
+            // vertex 0 has positive area.
+            P q{}; q.nv = 6;
+            const int id = (int)polys.size();
+            q.v[0] = vid(x + 1, z);     q.v[1] = vid(x, z);         q.v[2] = vid(x, z + 1);
+            q.v[3] = vid(x + 1, z + 1); q.v[4] = vid(x + 2, z + 1); q.v[5] = vid(x + 2, z);
+            const int ecx[6] = {x, x, x, x + 1, x + 1, x + 1};
+            const int esd[6] = {3, 0, 1, 1, 2, 3};
+            for (int e = 0; e < 6; ++e) { q.nei[e] = -1; q.cx[e] = ecx[e]; q.cz[e] = z; q.side[e] = esd[e]; own(ecx[e], z, esd[e], id); }
+            polys.push_back(q);
+          } else if (r < p.hex_frac + p.tri_frac) {
+            const int id = (int)polys.size();
+            P a{}, b{}; a.nv = b.nv = 3;
+            for (int e = 0; e < 6; ++e) { a.nei[e] = b.nei[e] = -1; a.side[e] = b.side[e] = -1; }
+            if (rng.next() & 1) {
+              a.v[0] = vid(x, z); a.v[1] = vid(x, z + 1); a.v[2] = vid(x + 1, z + 1);
+              a.side[0] = 0; a.side[1] = 1; a.nei[2] = id + 1;
+              b.v[0] = vid(x, z); b.v[1] = vid(x + 1, z + 1); b.v[2] = vid(x + 1, z);
+              b.nei[0] = id; b.side[1] = 2; b.side[2] = 3;
+            } else {
+              a.v[0] = vid(x, z); a.v[1] = vid(x, z + 1); a.v[2] = vid(x + 1, z);
+              a.side[0] = 0; a.nei[1] = id + 1; a.side[2] = 3;
+              b.v[0] = vid(x, z + 1); b.v[1] = vid(x + 1, z + 1); b.v[2] = vid(x + 1, z);
+              b.side[0] = 1; b.side[1] = 2; b.nei[2] = id;
+            }
+            for (int e = 0; e < 3; ++e) {
+              a.cx[e] = b.cx[e] = x; a.cz[e] = b.cz[e] = z;
+              if (a.side[e] >= 0) own(x, z, a.side[e], id);
+              if (b.side[e] >= 0) own(x, z, b.side[e], id + 1);
+            }
+            polys.push_back(a);
+            polys.push_back(b);
+          } else {
+            P q{}; q.nv = 4;
+            const int id = (int)polys.size();
+            q.v[0] = vid(x, z); q.v[1] = vid(x, z + 1); q.v[2] = vid(x + 1, z + 1); q.v[3] = vid(x + 1, z);
+            for (int e = 0; e < 4; ++e) { q.nei[e] = -1; q.cx[e] = x; q.cz[e] = z; q.side[e] = e; own(x, z, e, id); }
+            polys.push_back(q);
+          }
+        }
+      if (polys.empty()) continue;  // a tile without floor is not stored
+      if (polys.size() > 0x7fff) return fail(BPSX_E_INVAL, "gen_scene: more than 32767 polygons in a tile; use more tiles or larger cells");
+      if (verts.size() / 3 >= 0xffff) return fail(BPSX_E_INVAL, "gen_scene: too many vertices in a tile");
+      const int np = (int)polys.size();
+      std::vector<uint16_t> pk((size_t)np * 12, 0xffff);
+      std::vector<uint16_t> flags((size_t)np, kPolyFlagWalk);
+      std::vector<uint8_t> areas((size_t)np, 0);
+      for (int i = 0; i < np; ++i) {
+        P& q = polys[i];
+        for (int e = 0; e < q.nv; ++e) {
+          pk[(size_t)i * 12 + e] = (uint16_t)q.v[e];
+          uint16_t code = 0xffff;
+          if (q.nei[e] >= 0) {
+            code = (uint16_t)q.nei[e];
+          } else if (q.side[e] >= 0) {
+            const int ax = q.cx[e] + odx[q.side[e]], az = q.cz[e] + odz[q.side[e]];
+            if (g.in(ax, az) && g.get(ax, az)) {
+              if (ax >= x0 && ax < x1 && az >= z0 && az < z1) code = (uint16_t)sidePoly[((size_t)az * nx + ax) * 4 + ((q.side[e] + 2) & 3)];
+              else code = (uint16_t)(0x8000 | q.side[e]);  // portal: 0 x-, 1 z+, 2 x+, 3 z-
+            }
+          }
+          pk[(size_t)i * 12 + 6 + e] = code;
+        }
       }
-      pk[(size_t)i * 12 + 6 + e] = nei >= 0 ? (uint16_t)nei : 0xffff;
+      bpsx_tile_desc d{};
+      d.verts = verts.data();
+      d.vert_count = (uint32_t)(verts.size() / 3);
+      d.polys = pk.data();
+      d.poly_flags = flags.data();
+      d.poly_areas = areas.data();
+      d.poly_count = (uint32_t)np;
+      d.nvp = 6;
+      d.walkable_height = 0.88f;
+      d.walkable_radius = 0.18f;
+      d.walkable_climb = 0.2f;
+      d.cs = kCs; d.ch = kCh;
+      d.bmin[0] = p.origin[0] + (float)(x0 * cell) * kCs; d.bmin[1] = p.origin[1]; d.bmin[2] = p.origin[2] + (float)(z0 * cell) * kCs;
+      d.bmax[0] = d.bmin[0] + (float)(tw * cell) * kCs;
+      d.bmax[1] = p.origin[1] + 1.0f;
+      d.bmax[2] = d.bmin[2] + (float)(th * cell) * kCs;
+      d.tile_x = tx; d.tile_y = tz; d.tile_layer = 0;
+      d.build_bv_tree = 1;
+      std::vector<uint8_t> tile;
+      const int rc = pack_tile(d, tile);
+      if (rc) return rc;
+      maxPolys = std::max(maxPolys, (uint32_t)np);
+      tiles.push_back(std::move(tile));
     }
-  }
-  bpsx_tile_desc d{};
-  d.verts = verts.data();
-  d.vert_count = (uint32_t)(verts.size() / 3);
-  d.polys = pk.data();
-  d.poly_flags = flags.data();
-  d.poly_areas = areas.data();
-  d.poly_count = (uint32_t)np;
-  d.nvp = 6;
-  d.walkable_height = 0.88f;
-  d.walkable_radius = 0.18f;
-  d.walkable_climb = 0.2f;
-  d.cs = kCs; d.ch = kCh;
-  d.bmin[0] = p.origin[0]; d.bmin[1] = p.origin[1]; d.bmin[2] = p.origin[2];
-  d.bmax[0] = p.origin[0] + (float)(nx * cell) * kCs;
-  d.bmax[1] = p.origin[1] + 1.0f;
-  d.bmax[2] = p.origin[2] + (float)(nz * cell) * kCs;
-  d.build_bv_tree = 1;
-  std::vector<uint8_t> tile;
-  int rc = pack_tile(d, tile);
-  if (rc) return rc;
-  const uint8_t* tp = tile.data();
-  const size_t ts = tile.size();
+  if (tiles.empty()) return fail(BPSX_E_INVAL, "gen_scene: no walkable cells");
+  std::vector<const uint8_t*> tp;
+  std::vector<size_t> ts;
+  for (auto& t : tiles) { tp.push_back(t.data()); ts.push_back(t.size()); }
   uint8_t* o = nullptr; size_t os = 0;
-  rc = bpsx_pack_mset(&tp, &ts, 1, d.bmin, d.bmax[0] - d.bmin[0], d.bmax[2] - d.bmin[2], 1, (uint32_t)np, &o, &os);
+  const float tileW = (float)(tw * cell) * kCs, tileH = (float)(th * cell) * kCs;
+  const int rc = bpsx_pack_mset(tp.data(), ts.data(), (uint32_t)tiles.size(), p.origin, tileW, tileH, (uint32_t)tiles.size(),
+                                maxPolys, &o, &os);
   if (rc) return rc;
   mset.assign(o, o + os);
   free(o);

@@ -44,7 +44,9 @@ int parse_navmesh(const uint8_t* b, size_t n, HostScene* out) {
     off += (size_t)cur.dataSize;
   }
   if (tiles == 0) return fail(BPSX_E_INVAL, "navmesh: holds no tile");
-  if (tiles > 1) return fail(BPSX_E_UNSUPPORTED, "navmesh: multi-tile meshes are not supported yet");
+  // The reference cannot load these either: PathFinder builds polygon refs with salt and tile
+  // index swapped (PathFinder.cpp:67, 318), which only cancels out for a one-tile mesh.
+  if (tiles > 1) return fail(BPSX_E_UNSUPPORTED, "navmesh: multi-tile meshes are not supported (nor by the reference's PathFinder)");
 
   TileHeader h;
   memcpy(&h, tileData, sizeof(h));

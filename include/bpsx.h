@@ -201,8 +201,9 @@ typedef struct bpsx_scene_params {
   float tri_frac;                /* fraction of cells split into two triangles       */
   float hex_frac;                /* fraction of cells merged pairwise into hexagons  */
   float origin[3];               /* world position of the grid corner                */
+  uint32_t tiles_x, tiles_z;     /* split the floor into this many navmesh tiles (0 = 1) */
 } bpsx_scene_params;
-/* Generates one single-tile scene as MSET bytes (malloc'd, release with bpsx_free). */
+/* Generates one scene as MSET bytes (malloc'd, release with bpsx_free). */
 int bpsx_gen_scene(const bpsx_scene_params *p, uint8_t **out, size_t *out_size);
 /* Area-weighted random points on the walkable polygons of MSET bytes, host-only:
  * out_xyz f32[n][3]. Deterministic in seed. */

@@ -133,3 +133,10 @@ def test_error_paths(oracle, torch_cuda):
     with pytest.raises(RuntimeError):
         gen.rgba(0)
     gen.close()
+    from bps_nav_amd import scenes
+    four = scenes.gen_scene(scenes.BOX_ROOM, 5, 5, size_x=10.0, size_z=10.0, num_boxes=4, box_min=0.5, box_max=2.0,
+                            tiles_x=2, tiles_z=2)
+    with pytest.raises(RuntimeError, match="multi-tile"):
+        make_gen([(four, sc[0][1])], 8)
+    with pytest.raises(RuntimeError, match="magic"):
+        make_gen([(b"XXXX" + sc[0][0][4:], sc[0][1])], 8)

@@ -111,6 +111,48 @@ def test_packer_matches_reference_builder_bytes(reflib):
     assert bytes(buf[:size]) == mine
 
 
+def test_packer_matches_reference_builder_with_portal_edges(reflib):
+    """Tile-border portal codes (0x8000 | dir) go through the same neis mapping and link budget
+    as dtCreateNavMeshData (DetourNavMeshBuilder.cpp:381-396, 497-515)."""
+    if reflib is None:
+        pytest.skip("compiled reference not available outside the development container")
+    verts = np.array([[0, 0, 0], [0, 0, 20], [20, 0, 20], [20, 0, 0], [40, 0, 20], [40, 0, 0]], np.uint16)
+    pk = np.full((2, 12), 0xFFFF, np.uint16)
+    pk[0, :4] = (0, 1, 2, 3)
+    pk[0, 6:10] = (0x8000, 0x8001, 1, 0x8003)      # x-, z+ portals, neighbour 1, z- portal
+    pk[1, :4] = (3, 2, 4, 5)
+    pk[1, 6:10] = (0, 0x8001, 0x8002, 0xFFFF)      # neighbour 0, z+ portal, x+ portal, wall
+    bmin, bmax = np.array([0, 0, 0], np.float32), np.array([2, 1, 1], np.float32)
+    mine = scenes.pack_tile(verts, pk, bmin=tuple(bmin), bmax=tuple(bmax))
+    buf = np.zeros(len(mine) + 1024, np.uint8)
+    size = reflib.L.bpo_ref_create_tile(verts.reshape(-1), 6, pk.reshape(-1), np.ones(2, np.uint16), np.zeros(2, np.uint8),
+                                        2, 6, 0.88, 0.18, 0.2, bmin, bmax, 0.05, 0.05, buf, len(buf))
+    assert size == len(mine) and bytes(buf[:size]) == mine
+
+
+def test_generator_can_tile_a_scene():
+    one = scenes.gen_scene(scenes.BOX_ROOM, 5, 5, size_x=10.0, size_z=10.0, num_boxes=4, box_min=0.5, box_max=2.0)
+    four = scenes.gen_scene(scenes.BOX_ROOM, 5, 5, size_x=10.0, size_z=10.0, num_boxes=4, box_min=0.5, box_max=2.0,
+                            tiles_x=2, tiles_z=2)
+    assert struct.unpack_from("<i", one, 8)[0] == 1 and struct.unpack_from("<i", four, 8)[0] == 4
+    # same floor: the polygon counts of the four tiles add up to the single tile's
+    off, total = 40, 0
+    for _ in range(4):
+        ref, size = struct.unpack_from("<Ii", four, off)
+        total += struct.unpack_from("<i", four, off + 8 + 24)[0]
+        off += 8 + size
+    assert off == len(four) and total == struct.unpack_from("<i", one, 48 + 24)[0]
+
+
+def test_oracle_rejects_multi_tile_meshes(oracle):
+    # the reference's PathFinder is undefined on them (refs built with salt and tile swapped,
+    # PathFinder.cpp:67, 318), so neither the oracle nor the engine accepts them
+    four = scenes.gen_scene(scenes.BOX_ROOM, 5, 5, size_x=10.0, size_z=10.0, num_boxes=4, box_min=0.5, box_max=2.0,
+                            tiles_x=2, tiles_z=2)
+    with pytest.raises(RuntimeError, match="multi-tile"):
+        bpo.Nav(oracle, four)
+
+
 def test_packed_tile_matches_fixture_bytes():
     # pins the packer (tile layout, BV tree, MSET header) where the reference builder is absent:
     # the fixture's navmesh bytes were loaded and queried by the compiled reference
