@@ -37,6 +37,18 @@ struct alignas(128) PolyRec {
 };
 static_assert(sizeof(PolyRec) == 128, "PolyRec must be one cache line");
 
+// What A* needs of one polygon edge: where a path crossing it is taken to pass (the midpoint
+// of the portal, getEdgeMidPoint in DetourNavMeshQuery.cpp:2352-2381, computed once at upload
+// with the same float operations) and which polygon lies behind it.  Six of them per polygon,
+// so lane j of a wavefront fetches edge j of the expanded polygon with one 16-byte load.
+struct AEdge {
+  float mid[3];
+  uint32_t nb;   // polygon index behind the edge if the search may enter it (internal link to
+                 // a polygon that passes the query filter), else kNoNb
+};
+static_assert(sizeof(AEdge) == 16, "AEdge");
+constexpr uint32_t kNoNb = 0xffffu;
+
 // dtBVNode repacked at upload: same quantised bounds; a leaf carries its polygon index, an
 // internal node carries Detour's escape offset (for the in-order walk) and the index of its
 // right child (its left child is the next node), so a wavefront can descend level by level.
@@ -95,6 +107,7 @@ constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentReuse = 4u, kAgentSk
 
 struct NavData {
   const PolyRec* polys;
+  const AEdge* aedges;     // [polygon][kNvp]
   const BVNodeDev* bv;
   const uint8_t* dtris;    // [.][4]
   const float* dverts;     // [.][3]
@@ -102,14 +115,14 @@ struct NavData {
   const float* episodes;   // [.][10]
 };
 
-// A* node of the per-slot pool (dtNode, DetourNode.h:36-45): 32 bytes.
+// A* node of the per-slot pool (dtNode, DetourNode.h:36-45) as spilled to HBM: 32 bytes.
 struct ANode {
   float pos[3];
   float cost;
   float total;
-  uint32_t pidx;   // 1-based parent node index, 0 = none
-  uint32_t flags;  // 1 open, 2 closed
-  uint32_t id;     // polygon index within the scene
+  uint32_t link;   // polygon index within the scene (bits 0-14) | next node of the hash chain << 16
+  uint32_t state;  // flags (1 open, 2 closed) | 1-based parent node index << 2
+  uint32_t pad;
 };
 static_assert(sizeof(ANode) == 32, "ANode");
 
@@ -122,7 +135,6 @@ struct HeapEntry {
 struct alignas(128) GeoSlot {
   ANode nodes[kMaxNodes];
   HeapEntry heap_spill[kMaxNodes];
-  uint16_t next[kMaxNodes];          // hash chains of the spilled nodes
 };
 
 struct GeoQuery {

@@ -53,6 +53,7 @@ struct bpsx_sim {
   uint32_t num_groups = 1, envs_per_group = 0;
   // navmesh arrays
   PolyRec* d_polys = nullptr;
+  AEdge* d_aedges = nullptr;
   BVNodeDev* d_bv = nullptr;
   uint8_t* d_dtris = nullptr;
   float* d_dverts = nullptr;
@@ -157,6 +158,7 @@ int bpsx_finalize(bpsx_sim* sim) {
   if (npoly > 0xfffffff0ull || ntri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
   int rc;
   if ((rc = sim->alloc(&sim->d_polys, npoly))) return rc;
+  if ((rc = sim->alloc(&sim->d_aedges, npoly * kNvp))) return rc;
   if ((rc = sim->alloc(&sim->d_bv, nbv))) return rc;
   if ((rc = sim->alloc(&sim->d_dtris, ntri * 4))) return rc;
   if ((rc = sim->alloc(&sim->d_dverts, ndv * 3))) return rc;
@@ -165,6 +167,7 @@ int bpsx_finalize(bpsx_sim* sim) {
   std::vector<SceneDev> sd;
   for (auto& s : sim->scenes) {
     HIP_TRY(hipMemcpy(sim->d_polys + s.dev.poly_base, s.polys.data(), s.polys.size() * sizeof(PolyRec), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(sim->d_aedges + (size_t)s.dev.poly_base * kNvp, s.aedges.data(), s.aedges.size() * sizeof(AEdge), hipMemcpyHostToDevice));
     if (!s.bv.empty())
       HIP_TRY(hipMemcpy(sim->d_bv + s.dev.bv_base, s.bv.data(), s.bv.size() * sizeof(BVNodeDev), hipMemcpyHostToDevice));
     sd.push_back(s.dev);
@@ -180,7 +183,7 @@ int bpsx_finalize(bpsx_sim* sim) {
     }
   }
   HIP_TRY(hipMemcpy(sim->d_scenes, sd.data(), sd.size() * sizeof(SceneDev), hipMemcpyHostToDevice));
-  sim->nav = NavData{sim->d_polys, sim->d_bv, sim->d_dtris, sim->d_dverts, sim->d_scenes, sim->d_episodes};
+  sim->nav = NavData{sim->d_polys, sim->d_aedges, sim->d_bv, sim->d_dtris, sim->d_dverts, sim->d_scenes, sim->d_episodes};
 
   // ---- agent state
   const size_t N = sim->cfg.num_environments;
@@ -210,7 +213,7 @@ int bpsx_finalize(bpsx_sim* sim) {
   // ---- A* wavefronts: as many as the LDS of the device holds at once, not one per agent
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, sim->cfg.gpu_id));
-  uint32_t per_cu = 9;  // 160 KB of LDS per CU / 17 KB per A* wavefront
+  uint32_t per_cu = geodesic_blocks_per_cu();
   if (const char* e = getenv("BPSX_GEO_WAVES_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e));
   uint32_t blocks = (uint32_t)prop.multiProcessorCount * per_cu;
   if (blocks > 2 * sim->envs_per_group) blocks = 2 * sim->envs_per_group;

@@ -4,17 +4,19 @@
 //
 // Execution model: one wavefront (64 lanes) owns one query at a time and pulls the next from
 // a shared queue when done.  The whole working set of A* lives in LDS: the open list (a binary
-// heap whose pops and pushes are done by all lanes at once, see HeapOps), the hash heads and
-// chains of the node pool, and the first kNodesLds nodes; only nodes beyond that and heap
-// entries beyond kHeapLds spill to a per-wavefront scratch slot in HBM.  Per expanded node the
-// only HBM traffic is the polygon's 128-byte record.  Lane j of the wavefront handles edge j of
-// the expanded polygon (node lookup, portal midpoint, cost); heap updates are then applied in
-// edge order, which is what makes the result identical to the sequential algorithm, ties
-// included.
+// heap), the hash heads and chains of the node pool, and the first kNodesLds nodes; only
+// nodes beyond that and heap entries beyond kHeapLds spill to a per-wavefront slot in HBM.
+// A query runs the LDS-only instantiation of the loop until its pool or heap could outgrow
+// LDS within one more expansion, then carries on in the spilling instantiation.  Per expanded
+// node the only HBM traffic is the polygon's six 16-byte edge records: lane j of the wavefront
+// handles edge j (node lookup, cost, heuristic); heap updates are then applied in edge order,
+// which is what makes the result identical to the sequential algorithm, ties included.
+// Everything that is the same for all lanes (heap walks, counters, the expanded node) is kept
+// in scalar registers and branches on the scalar unit.
 //
 // Reference semantics followed: DetourNavMeshQuery.cpp:945-1178 (findPath, getPathToNode),
-// :1661-1696, 1765-1994 (appendVertex, findStraightPath), :2279-2349 (getPortalPoints);
-// DetourNode.cpp:50-200 (node pool, heap order); PathFinder.cpp:473-541.
+// :1661-1696, 1765-1994 (appendVertex, findStraightPath), :2279-2381 (getPortalPoints,
+// getEdgeMidPoint); DetourNode.cpp:50-200 (node pool, heap order); PathFinder.cpp:473-541.
 #pragma once
 #include "nav_device.h"
 
@@ -26,8 +28,14 @@ namespace bpsx {
 #define PHASE_MARK(k) do { } while (0)
 #endif
 
-constexpr int kNodesLds = 512;   // nodes kept in LDS per query
-constexpr int kHeapLds = 384;    // open-list entries kept in LDS per query
+#ifndef BPSX_NODES_LDS
+#define BPSX_NODES_LDS 512
+#endif
+#ifndef BPSX_HEAP_LDS
+#define BPSX_HEAP_LDS 256
+#endif
+constexpr int kNodesLds = BPSX_NODES_LDS;   // nodes kept in LDS per query
+constexpr int kHeapLds = BPSX_HEAP_LDS;     // open-list entries kept in LDS per query
 constexpr int kHashSize = 512;
 
 BPSX_DEV void wave_sync() {
@@ -37,6 +45,7 @@ BPSX_DEV void wave_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 BPSX_DEV int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
+BPSX_DEV float uniform_f(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 BPSX_DEV float lane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
 BPSX_DEV int lane_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
 
@@ -45,8 +54,8 @@ struct GeoLds {
   float n_total[kNodesLds];
   float n_cost[kNodesLds];
   float n_pos[3][kNodesLds];
-  uint32_t n_meta[kNodesLds];      // id:15 | flags:2 << 15 | pidx:12 << 17
-  uint16_t n_next[kNodesLds];
+  uint32_t n_link[kNodesLds];      // polygon index (bits 0-14) | next node of the hash chain << 16
+  uint16_t n_state[kNodesLds];     // flags (1 open, 2 closed) | 1-based parent node index << 2
   uint16_t first[kHashSize];
   HeapEntry heap[kHeapLds];
 };
@@ -55,19 +64,16 @@ struct FunnelLds {
   float portals[kMaxPath][6];
   uint16_t corridor[kMaxPath];
 };
-static_assert(sizeof(FunnelLds) <= offsetof(GeoLds, n_meta), "funnel scratch must stay clear of the node links");
+static_assert(sizeof(FunnelLds) <= offsetof(GeoLds, n_link), "funnel scratch must stay clear of the node links");
 
-BPSX_DEV uint32_t meta_pack(uint32_t id, uint32_t flags, uint32_t pidx) { return id | (flags << 15) | (pidx << 17); }
-BPSX_DEV uint32_t meta_id(uint32_t m) { return m & 0x7fffu; }
-BPSX_DEV uint32_t meta_flags(uint32_t m) { return (m >> 15) & 3u; }
-BPSX_DEV uint32_t meta_pidx(uint32_t m) { return m >> 17; }
+constexpr uint32_t kChainEnd = 0xffffu;
+BPSX_DEV uint32_t link_id(uint32_t l) { return l & 0x7fffu; }
+BPSX_DEV uint32_t link_next(uint32_t l) { return l >> 16; }
+BPSX_DEV uint32_t state_flags(uint32_t s) { return s & 3u; }
+BPSX_DEV uint32_t state_pidx(uint32_t s) { return s >> 2; }
 
-struct NodeVal {
-  float pos[3];
-  float cost, total;
-  uint32_t meta;
-};
-
+// Accessors take the instantiation's spill switch S: with S false every index is known to be
+// inside LDS and no address-space branch is generated.
 struct GeoWave {
   GeoLds* L;
   GeoSlot* ws;
@@ -76,170 +82,253 @@ struct GeoWave {
   int nodeCount;
 
   // ---------------------------------------------------------------- node pool
-  BPSX_DEV uint32_t node_meta(int i) const {
-    if (i < kNodesLds) return L->n_meta[i];
-    const ANode& n = ws->nodes[i];
-    return meta_pack(n.id, n.flags, n.pidx);
+  template <bool S> BPSX_DEV uint32_t link(int i) const { return (!S || i < kNodesLds) ? L->n_link[i] : ws->nodes[i].link; }
+  template <bool S> BPSX_DEV void set_link(int i, uint32_t v) const {
+    if (!S || i < kNodesLds) L->n_link[i] = v;
+    else ws->nodes[i].link = v;
   }
-  BPSX_DEV NodeVal node_load(int i) const {
-    NodeVal v;
-    if (i < kNodesLds) {
-      v.pos[0] = L->n_pos[0][i]; v.pos[1] = L->n_pos[1][i]; v.pos[2] = L->n_pos[2][i];
-      v.cost = L->n_cost[i]; v.total = L->n_total[i]; v.meta = L->n_meta[i];
-    } else {
-      const ANode n = ws->nodes[i];
-      v.pos[0] = n.pos[0]; v.pos[1] = n.pos[1]; v.pos[2] = n.pos[2];
-      v.cost = n.cost; v.total = n.total; v.meta = meta_pack(n.id, n.flags, n.pidx);
-    }
-    return v;
+  template <bool S> BPSX_DEV uint32_t state(int i) const { return (!S || i < kNodesLds) ? (uint32_t)L->n_state[i] : ws->nodes[i].state; }
+  template <bool S> BPSX_DEV void set_state(int i, uint32_t v) const {
+    if (!S || i < kNodesLds) L->n_state[i] = (uint16_t)v;
+    else ws->nodes[i].state = v;
   }
-  BPSX_DEV void node_store(int i, const NodeVal& v) const {
-    if (i < kNodesLds) {
-      L->n_pos[0][i] = v.pos[0]; L->n_pos[1][i] = v.pos[1]; L->n_pos[2][i] = v.pos[2];
-      L->n_cost[i] = v.cost; L->n_total[i] = v.total; L->n_meta[i] = v.meta;
-    } else {
-      ANode n;
-      n.pos[0] = v.pos[0]; n.pos[1] = v.pos[1]; n.pos[2] = v.pos[2];
-      n.cost = v.cost; n.total = v.total;
-      n.id = meta_id(v.meta); n.flags = meta_flags(v.meta); n.pidx = meta_pidx(v.meta);
-      ws->nodes[i] = n;
-    }
-  }
-  BPSX_DEV void node_set_meta(int i, uint32_t m) const {
-    if (i < kNodesLds) L->n_meta[i] = m;
-    else { ws->nodes[i].flags = meta_flags(m); ws->nodes[i].pidx = meta_pidx(m); ws->nodes[i].id = meta_id(m); }
-  }
-  BPSX_DEV int node_next(int i) const { return i < kNodesLds ? L->n_next[i] : ws->next[i]; }
-  static BPSX_DEV uint32_t hash(uint32_t a) {
-    a ^= a >> 16; a *= 0x7feb352du; a ^= a >> 15; a *= 0x846ca68bu; a ^= a >> 16;
-    return a & (kHashSize - 1);
-  }
+  static BPSX_DEV uint32_t hash(uint32_t ip) { return (__umul24(ip, 0x9e3779u) >> 9) & (kHashSize - 1); }
   BPSX_DEV void clear() {
-    for (int i = lane; i < kHashSize; i += 64) L->first[i] = 0xffff;
+    for (int i = lane; i < kHashSize; i += 64) L->first[i] = (uint16_t)kChainEnd;
     heapSize = 0;
     nodeCount = 0;
     wave_sync();
   }
-  // node index of polygon ip, or -1 (any lane, independently)
-  BPSX_DEV int find(uint32_t ip) const {
-    for (int i = L->first[hash(ip)]; i != 0xffff; i = node_next(i))
-      if (meta_id(node_meta(i)) == ip) return i;
+  // node index of polygon ip, or -1 (any lane, independently); one LDS access per chain step
+  template <bool S> BPSX_DEV int find(uint32_t ip, uint32_t bucket) const {
+    for (uint32_t i = L->first[bucket]; i != kChainEnd;) {
+      const uint32_t l = link<S>((int)i);
+      if (link_id(l) == ip) return (int)i;
+      i = link_next(l);
+    }
     return -1;
-  }
-  // Links node i (already counted in nodeCount) into the hash; executed by one lane.
-  BPSX_DEV void link(int i, uint32_t ip) const {
-    const uint32_t b = hash(ip);
-    const uint16_t head = L->first[b];
-    if (i < kNodesLds) L->n_next[i] = head;
-    else ws->next[i] = head;
-    L->first[b] = (uint16_t)i;
   }
 
   // ---------------------------------------------------------------- open list
-  BPSX_DEV HeapEntry hget(int i) const { return i < kHeapLds ? L->heap[i] : ws->heap_spill[i]; }
-  BPSX_DEV float ht(int i) const { return hget(i).total; }
-  BPSX_DEV int hn(int i) const { return (int)hget(i).node; }
-  BPSX_DEV void hset(int i, float t, int n) const {
+  // The heap is walked with wave-uniform indices: every lane issues the same LDS access and the
+  // values are moved to scalar registers, so the loops below branch on the scalar unit and cost
+  // a handful of vector instructions per level.
+  template <bool S> BPSX_DEV HeapEntry hget(int i) const { return (!S || i < kHeapLds) ? L->heap[i] : ws->heap_spill[i]; }
+  template <bool S> BPSX_DEV void hset(int i, float t, int n) const {
     const HeapEntry e{t, (uint32_t)n};
-    if (i < kHeapLds) L->heap[i] = e;
-    else ws->heap_spill[i] = e;
+    if (!S || i < kHeapLds) L->heap[i] = e;   // all lanes store the same value to the same address
+    else if (lane == 0) ws->heap_spill[i] = e;
   }
-  // dtNodeQueue::bubbleUp from index i0 with entry (t, n), all ancestors looked at at once:
-  // along a leaf-to-root path the keys never increase, so the ancestors that are greater than
-  // t form a prefix; they each move one level down and the entry lands above them.
-  BPSX_DEV void bubble_up(int i0, float t, int n) const {
-    // lane d holds ancestor a_d = ((i0 + 1) >> d) - 1 (a_0 = i0; -1 once past the root)
-    const int a = lane <= 12 ? ((i0 + 1) >> lane) - 1 : -1;
-    const bool valid = lane >= 1 && a >= 0;
-    float at = 0;
-    int an = 0;
-    if (valid) { const HeapEntry e = hget(a); at = e.total; an = (int)e.node; }
-    const unsigned long long gt = __ballot(valid && at > t);
-    const int m = __popcll(gt);  // ancestors 1..m move down
-    wave_sync();
-    // lane d (1..m) writes its ancestor's entry one level down, into a_{d-1}
-    const int child = lane >= 1 && lane <= 13 ? ((i0 + 1) >> (lane - 1)) - 1 : 0;
-    if (lane >= 1 && lane <= m) hset(child, at, an);
-    if (lane == m) hset(lane == 0 ? i0 : a, t, n);
+  // dtNodeQueue::bubbleUp from index i with entry (t, n)
+  template <bool S> BPSX_DEV void bubble_up(int i, float t, int n) const {
+    while (i > 0) {
+      const int parent = (i - 1) >> 1;
+      const HeapEntry pe = hget<S>(parent);
+      const float pt = uniform_f(pe.total);
+      if (!(pt > t)) break;
+      hset<S>(i, pt, uniform_i((int)pe.node));
+      i = parent;
+    }
+    hset<S>(i, t, n);
     wave_sync();
   }
-  BPSX_DEV void push(float t, int n) {
+  template <bool S> BPSX_DEV void push(float t, int n) {
     heapSize++;
-    bubble_up(heapSize - 1, t, n);
+    bubble_up<S>(heapSize - 1, t, n);
   }
-  BPSX_DEV void modify(int n, float t) const {
+  template <bool S> BPSX_DEV void modify(int n, float t) const {
     int found = -1;
     for (int base = 0; base < heapSize; base += 64) {
       const int i = base + lane;
-      const unsigned long long m = __ballot(i < heapSize && hn(i) == n);
+      const unsigned long long m = __ballot(i < heapSize && (int)hget<S>(i).node == n);
       if (m) { found = base + (__ffsll((long long)m) - 1); break; }
     }
-    if (found >= 0) bubble_up(found, t, n);
+    if (found >= 0) bubble_up<S>(found, t, n);
   }
-  // dtNodeQueue::pop: the hole left by the root travels down along the smaller children to a
-  // leaf, then the former last entry bubbles up from there.  The route depends only on the
-  // heap's contents, so lanes evaluate "which child is smaller" for 63 nodes of a subtree at
-  // once and the route is then read off with scalar lane reads; the entries on the route that
-  // are not greater than the re-inserted entry shift up one level, it lands below them, and
-  // the rest of the route stays as it was.
-  BPSX_DEV int pop() {
-    const int top = hn(0);
+  // dtNodeQueue::pop (the caller has read the root). The reference moves the hole left by the
+  // root down to a leaf along the smaller children and then bubbles the former last entry up
+  // from there; along that route keys never decrease, so the entry ends up above the first
+  // route element that is greater than it: the walk can stop there, nothing below moves.
+  template <bool S> BPSX_DEV void pop() {
     heapSize--;
     const int size = heapSize;
-    if (size == 0) return top;
-    const HeapEntry lastE = hget(size);
-    const float lt = lastE.total;
-    const int ln = (int)lastE.node;
-    // route entries are collected one per lane: lane d keeps the d-th node of the route
-    float myT = 0;
-    int myN = 0, myIdx = -1, myParent = -1;
-    int depth = 0;   // number of route nodes below the root found so far (uniform)
-    int root = 0;    // root of the subtree being resolved (uniform)
+    if (size == 0) return;
+    const HeapEntry lastE = hget<S>(size);
+    const float lt = uniform_f(lastE.total);
+    const int ln = uniform_i((int)lastE.node);
+    int i = 0;
     for (;;) {
-      // lane t (< 63) looks at node (root+1 << lvl) - 1 + off of the subtree, lvl = floor(log2(t+1))
-      const int t1 = lane + 1;
-      const int lvl = 31 - __clz(t1);
-      const int node = ((root + 1) << lvl) - 1 + (t1 - (1 << lvl));
-      int choice = -1;
-      float ct = 0;
-      int cn = 0;
-      if (lane < 63) {
-        const int c1 = 2 * node + 1;
-        if (c1 < size) {
-          const HeapEntry e1 = hget(c1);
-          ct = e1.total; cn = (int)e1.node; choice = c1;
-          if (c1 + 1 < size) {
-            const HeapEntry e2 = hget(c1 + 1);
-            if (ct > e2.total) { ct = e2.total; cn = (int)e2.node; choice = c1 + 1; }
-          }
-        }
-      }
-      // follow the choices from the subtree's root: relative lane r -> 2r+1 or 2r+2
-      int r = 0, cur = root;
-      bool more = false;
-      for (int s = 0; s < 6; ++s) {
-        const int c = lane_i(choice, r);
-        if (c < 0) break;
-        const float tt = lane_f(ct, r);
-        const int nn = lane_i(cn, r);
-        depth++;
-        if (lane == depth) { myT = tt; myN = nn; myIdx = c; myParent = cur; }
-        r = 2 * r + 1 + (c - (2 * cur + 1));
-        cur = c;
-        if (r >= 63) { more = true; break; }
-      }
-      if (!more) break;
-      root = cur;
+      const int c = 2 * i + 1;
+      if (c >= size) break;
+      const bool two = c + 1 < size;
+      // odd lanes fetch the right child, even lanes the left one: one LDS instruction
+      const HeapEntry e = hget<S>(c + ((two && (lane & 1)) ? 1 : 0));
+      const float t0 = lane_f(e.total, 0), t1 = lane_f(e.total, 1);
+      const bool right = two && t0 > t1;
+      const float tc = right ? t1 : t0;
+      if (!(tc <= lt)) break;
+      const int nc = right ? lane_i((int)e.node, 1) : lane_i((int)e.node, 0);
+      hset<S>(i, tc, nc);
+      i = c + (right ? 1 : 0);
     }
-    const unsigned long long le = __ballot(lane >= 1 && lane <= depth && myT <= lt);
-    const int j = __popcll(le);  // route entries 1..j shift up, the re-inserted entry lands at route[j]
+    hset<S>(i, lt, ln);
     wave_sync();
-    if (lane >= 1 && lane <= j) hset(myParent, myT, myN);
-    if (lane == j) hset(j == 0 ? 0 : myIdx, lt, ln);
-    wave_sync();
-    return top;
   }
 };
+
+struct AstarState {
+  int lastBest;
+  float lastBestCost;
+  bool outOfNodes;
+};
+enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrow = 2 };
+
+// The expansion loop of findPath. S = false: all nodes and heap entries are in LDS; returns
+// kAstarGrow before an expansion that could need more than LDS holds.
+template <bool S>
+BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
+#ifdef BPSX_PHASE_TIMING
+                              , unsigned long long* phase_acc, unsigned long long& phase_t0
+#endif
+                              ) {
+  const int lane = g.lane;
+  GeoLds* L = g.L;
+  const float H_SCALE = 0.999f;
+  const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
+  while (g.heapSize > 0) {
+    if (!S && (g.nodeCount > kNodesLds - kNvp || g.heapSize > kHeapLds - kNvp)) return kAstarGrow;
+    // the node about to be popped is the root: fetch its edges while the heap is repaired
+    const int bi = uniform_i((int)L->heap[0].node);
+    float b0, b1, b2, bcost;
+    uint32_t bestIp, pidx;
+    if (!S || bi < kNodesLds) {
+      b0 = L->n_pos[0][bi]; b1 = L->n_pos[1][bi]; b2 = L->n_pos[2][bi]; bcost = L->n_cost[bi];
+      bestIp = link_id((uint32_t)uniform_i((int)L->n_link[bi]));
+      pidx = state_pidx((uint32_t)uniform_i((int)L->n_state[bi]));
+    } else {
+      const ANode& n = g.ws->nodes[bi];
+      b0 = n.pos[0]; b1 = n.pos[1]; b2 = n.pos[2]; bcost = n.cost;
+      bestIp = link_id((uint32_t)uniform_i((int)n.link));
+      pidx = state_pidx((uint32_t)uniform_i((int)n.state));
+    }
+    uint32_t nb = kNoNb;
+    float m0 = 0, m1 = 0, m2 = 0;
+    if (lane < kNvp) {
+      const AEdge e = edges[bestIp * kNvp + lane];
+      nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
+    }
+    PHASE_MARK(0);
+    g.pop<S>();
+    PHASE_MARK(1);
+    g.set_state<S>(bi, 2u | (pidx << 2));   // open -> closed
+    if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
+    (*pops)++;
+    // a polygon reached through two edges of the same expansion: the second visit never
+    // changes the node (same position, same cost), so only the first edge counts
+    {
+      const uint32_t orig = nb;
+#pragma unroll
+      for (int k = 0; k < kNvp - 1; ++k) {
+        const uint32_t other = (uint32_t)lane_i((int)orig, k);
+        if (lane > k && other == orig) nb = kNoNb;
+      }
+    }
+    PHASE_MARK(2);
+    const uint32_t bucket = GeoWave::hash(nb);
+    int ni = -1;
+    if (nb != kNoNb) ni = g.find<S>(nb, bucket);
+    // the polygon the expanded node was reached from is not entered again
+    if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
+    PHASE_MARK(3);
+    // new nodes take consecutive indices in edge order; past the pool's end they are dropped
+    const unsigned long long need = __ballot(nb != kNoNb && ni < 0);
+    const bool isNew = (need >> lane) & 1ull;
+    if (need) {
+      const int rank = __popcll(need & ((1ull << lane) - 1ull));
+      if (isNew) {
+        const int idx = g.nodeCount + rank;
+        if (!S || idx < kMaxNodes) ni = idx;
+        else nb = kNoNb;
+      }
+      const int want = g.nodeCount + __popcll(need);
+      if (S && want > kMaxNodes) st.outOfNodes = true;
+      g.nodeCount = (!S || want < kMaxNodes) ? want : kMaxNodes;
+      // hash insertion by all new nodes at once; of two that share a bucket one store wins
+      // and the other lane goes round again behind it
+      bool pending = isNew && nb != kNoNb;
+      while (__ballot(pending)) {
+        if (pending) {
+          const uint32_t head = L->first[bucket];
+          g.set_link<S>(ni, nb | (head << 16));
+          L->first[bucket] = (uint16_t)ni;
+        }
+        wave_sync();
+        if (pending && L->first[bucket] == (uint16_t)ni) pending = false;
+        wave_sync();
+      }
+    }
+    PHASE_MARK(4);
+    bool update = false, wasOpen = false;
+    float total = 0, heuristic = 0;
+    if (nb != kNoNb) {
+      float p0 = m0, p1 = m1, p2 = m2, oldTotal = 0;
+      uint32_t fl = 0;
+      if (!isNew) {
+        if (!S || ni < kNodesLds) {
+          p0 = L->n_pos[0][ni]; p1 = L->n_pos[1][ni]; p2 = L->n_pos[2][ni];
+          oldTotal = L->n_total[ni]; fl = state_flags(L->n_state[ni]);
+        } else {
+          const ANode& n = g.ws->nodes[ni];
+          p0 = n.pos[0]; p1 = n.pos[1]; p2 = n.pos[2]; oldTotal = n.total; fl = state_flags(n.state);
+        }
+      }
+      const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
+      const float curCost = sqrtf(cx * cx + cy * cy + cz * cz) * 1.0f;
+      const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
+      const float toEnd = sqrtf(ex * ex + ey * ey + ez * ez);
+      float cost;
+      if (nb == endIp) {
+        cost = bcost + curCost + toEnd * 1.0f;
+        heuristic = 0;
+      } else {
+        cost = bcost + curCost;
+        heuristic = toEnd * H_SCALE;
+      }
+      total = cost + heuristic;
+      const bool worse = fl && total >= oldTotal;
+      if (!worse) {
+        update = true;
+        wasOpen = (fl & 1u) != 0;
+        const uint32_t ns = 1u | ((uint32_t)(bi + 1) << 2);   // open, parent = expanded node
+        if (!S || ni < kNodesLds) {
+          if (isNew) { L->n_pos[0][ni] = p0; L->n_pos[1][ni] = p1; L->n_pos[2][ni] = p2; }
+          L->n_cost[ni] = cost; L->n_total[ni] = total; L->n_state[ni] = (uint16_t)ns;
+        } else {
+          ANode& n = g.ws->nodes[ni];
+          if (isNew) { n.pos[0] = p0; n.pos[1] = p1; n.pos[2] = p2; }
+          n.cost = cost; n.total = total; n.state = ns;
+        }
+      }
+    }
+    wave_sync();
+    PHASE_MARK(5);
+    // ---- ordered phase: heap and "nearest so far" updates in edge order
+    unsigned long long upd = __ballot(update);
+    while (upd) {
+      const int src = __ffsll((long long)upd) - 1;
+      upd &= upd - 1;
+      const int node = lane_i(ni, src);
+      const float t = lane_f(total, src);
+      const float h = lane_f(heuristic, src);
+      const bool open = lane_i(wasOpen ? 1 : 0, src) != 0;
+      if (open) g.modify<S>(node, t);
+      else g.push<S>(t, node);
+      if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = node; }
+    }
+    PHASE_MARK(6);
+  }
+  return kAstarEmpty;
+}
 
 // Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
 // when the reference would report anything but plain DT_SUCCESS.
@@ -259,167 +348,47 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     return 1;
   }
   g.clear();
-  const float H_SCALE = 0.999f;
+  AstarState st;
   {
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
-    const float total = sqrtf(dx * dx + dy * dy + dz * dz) * H_SCALE;
+    const float total = sqrtf(dx * dx + dy * dy + dz * dz) * 0.999f;
     g.nodeCount = 1;
     if (lane == 0) {
-      NodeVal v;
-      v.pos[0] = startPos[0]; v.pos[1] = startPos[1]; v.pos[2] = startPos[2];
-      v.cost = 0; v.total = total; v.meta = meta_pack(startIp, 1u, 0u);
-      g.node_store(0, v);
-      g.link(0, startIp);
+      GeoLds* L = g.L;
+      L->n_pos[0][0] = startPos[0]; L->n_pos[1][0] = startPos[1]; L->n_pos[2][0] = startPos[2];
+      L->n_cost[0] = 0; L->n_total[0] = total;
+      L->n_state[0] = 1;   // open, no parent
+      L->n_link[0] = startIp | (kChainEnd << 16);
+      L->first[GeoWave::hash(startIp)] = 0;
     }
     wave_sync();
-    g.push(total, 0);
+    g.push<false>(total, 0);
+    st.lastBest = 0;
+    st.lastBestCost = total;
+    st.outOfNodes = false;
   }
-  int lastBest = 0;
-  float lastBestCost = g.L->n_total[0];
-  bool outOfNodes = false;
-  while (g.heapSize > 0) {
-    // the node about to be popped is the root: fetch its polygon while the heap is repaired
-    const int bi = uniform_i(g.hn(0));
-    const NodeVal best = g.node_load(bi);
-    const uint32_t bestIp = meta_id(best.meta);
-    const PolyRec* bp = &nav.polys[s.poly_base + bestIp];
-    uint32_t nbRaw = 0, nbWalk = 0;
-    float l0 = 0, l1 = 0, l2 = 0, r0 = 0, r1 = 0, r2 = 0;
-    const int nv = bp->nv;
-    if (lane < kNvp) {
-      nbRaw = bp->nei[lane];
-      nbWalk = bp->walk[lane];
-      l0 = bp->v[lane][0]; l1 = bp->v[lane][1]; l2 = bp->v[lane][2];
-      if (lane + 1 < kNvp) { r0 = bp->v[lane + 1][0]; r1 = bp->v[lane + 1][1]; r2 = bp->v[lane + 1][2]; }
-    }
-    const uint32_t pidx = meta_pidx(best.meta);
-    const uint32_t parentIp = pidx ? meta_id(g.node_meta((int)pidx - 1)) : kInvalidPoly;
-    PHASE_MARK(0);
-    g.pop();
-    PHASE_MARK(1);
-    if (lane == 0) g.node_set_meta(bi, meta_pack(bestIp, (meta_flags(best.meta) & ~1u) | 2u, pidx));
-    wave_sync();
-    if (bestIp == endIp) { lastBest = bi; break; }
-    (*pops)++;
-    // right end of edge j is vertex j+1, wrapping to vertex 0 on the last edge
-    {
-      const float w0 = lane_f(l0, 0), w1 = lane_f(l1, 0), w2 = lane_f(l2, 0);
-      if (lane + 1 >= nv) { r0 = w0; r1 = w1; r2 = w2; }
-    }
-    // ---- per-edge phase: lane j looks at edge j
-    uint32_t nb = kInvalidPoly;
-    if (lane < nv) {
-      const uint32_t w = (nbRaw & 0x8000u) ? 0u : nbRaw;
-      if (w && (w - 1) != parentIp && nbWalk) nb = w - 1;
-    }
-    // a polygon reached through two edges of the same expansion: the second visit never
-    // changes the node (same position, same cost), so only the first edge counts
-    {
-      const uint32_t orig = nb;
-#pragma unroll
-      for (int k = 0; k < kNvp - 1; ++k) {
-        const uint32_t other = (uint32_t)lane_i((int)orig, k);
-        if (lane > k && other == orig) nb = kInvalidPoly;
-      }
-    }
-    PHASE_MARK(2);
-    int ni = -1;
-    if (nb != kInvalidPoly) ni = g.find(nb);
-    PHASE_MARK(3);
-    // new nodes take consecutive indices in edge order; past the pool's end they are dropped
-    {
-      const unsigned long long need = __ballot(nb != kInvalidPoly && ni < 0);
-      if (need) {
-        const int rank = __popcll(need & ((1ull << lane) - 1ull));
-        const bool mine = (need >> lane) & 1ull;
-        if (mine) {
-          const int idx = g.nodeCount + rank;
-          if (idx < kMaxNodes) ni = idx;
-          else nb = kInvalidPoly;
-        }
-        const int want = g.nodeCount + __popcll(need);
-        if (want > kMaxNodes) outOfNodes = true;
-        g.nodeCount = want < kMaxNodes ? want : kMaxNodes;
-        // hash insertion one node at a time (two new nodes may share a bucket)
-        unsigned long long todo = need;
-        while (todo) {
-          const int src = __ffsll((long long)todo) - 1;
-          todo &= todo - 1;
-          if (lane == src && nb != kInvalidPoly) g.link(ni, nb);
-          wave_sync();
-        }
-        if (mine && nb != kInvalidPoly) {
-          NodeVal v;
-          v.pos[0] = v.pos[1] = v.pos[2] = 0; v.cost = 0; v.total = 0; v.meta = meta_pack(nb, 0u, 0u);
-          g.node_store(ni, v);
-        }
-      }
-    }
-    PHASE_MARK(4);
-    bool update = false;
-    float total = 0, heuristic = 0;
-    bool wasOpen = false;
-    if (nb != kInvalidPoly) {
-      NodeVal nn = g.node_load(ni);
-      uint32_t fl = meta_flags(nn.meta);
-      if (fl == 0) {
-        nn.pos[0] = (l0 + r0) * 0.5f;
-        nn.pos[1] = (l1 + r1) * 0.5f;
-        nn.pos[2] = (l2 + r2) * 0.5f;
-      }
-      const float cx = nn.pos[0] - best.pos[0], cy = nn.pos[1] - best.pos[1], cz = nn.pos[2] - best.pos[2];
-      const float curCost = sqrtf(cx * cx + cy * cy + cz * cz) * 1.0f;
-      const float ex = endPos[0] - nn.pos[0], ey = endPos[1] - nn.pos[1], ez = endPos[2] - nn.pos[2];
-      const float toEnd = sqrtf(ex * ex + ey * ey + ez * ez);
-      float cost;
-      if (nb == endIp) {
-        cost = best.cost + curCost + toEnd * 1.0f;
-        heuristic = 0;
-      } else {
-        cost = best.cost + curCost;
-        heuristic = toEnd * H_SCALE;
-      }
-      total = cost + heuristic;
-      const bool worse = (fl & 3u) && total >= nn.total;
-      if (!worse) {
-        update = true;
-        wasOpen = (fl & 1u) != 0;
-        nn.meta = meta_pack(nb, (fl & ~2u) | 1u, (uint32_t)bi + 1);
-        nn.cost = cost;
-        nn.total = total;
-        g.node_store(ni, nn);
-      }
-    }
-    wave_sync();
-    PHASE_MARK(5);
-    // ---- ordered phase: heap and "nearest so far" updates in edge order
-    unsigned long long upd = __ballot(update);
-    while (upd) {
-      const int src = __ffsll((long long)upd) - 1;
-      upd &= upd - 1;
-      const int node = lane_i(ni, src);
-      const float t = lane_f(total, src);
-      const float h = lane_f(heuristic, src);
-      const bool open = lane_i(wasOpen ? 1 : 0, src) != 0;
-      if (open) g.modify(node, t);
-      else g.push(t, node);
-      if (h < lastBestCost) { lastBestCost = h; lastBest = node; }
-    }
-    PHASE_MARK(6);
-  }
+  const AEdge* edges = nav.aedges + (size_t)s.poly_base * kNvp;
+#ifdef BPSX_PHASE_TIMING
+  AstarExit ex = astar_loop<false>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0);
+  if (ex == kAstarGrow) ex = astar_loop<true>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0);
+#else
+  AstarExit ex = astar_loop<false>(g, st, edges, endIp, endPos, pops);
+  if (ex == kAstarGrow) ex = astar_loop<true>(g, st, edges, endIp, endPos, pops);
+#endif
+  (void)ex;
+  const int lastBest = st.lastBest;
   // getPathToNode
   int length = 0;
-  for (int c = lastBest + 1; c; c = (int)meta_pidx(g.node_meta(c - 1))) length++;
-  const bool ok = length <= kMaxPath && meta_id(g.node_meta(lastBest)) == endIp && !outOfNodes;
+  for (int c = lastBest + 1; c; c = (int)state_pidx(g.state<true>(c - 1))) length++;
+  const bool ok = length <= kMaxPath && link_id(g.link<true>(lastBest)) == endIp && !st.outOfNodes;
   if (!ok) return 0;
-  // the corridor goes into LDS that overlays the nodes' cost and position arrays; the parent
-  // links (n_meta) are outside that region and stay readable while it is written
+  // the corridor goes into LDS that overlays the nodes' cost and position arrays; the links
+  // and parent indices are outside that region and stay readable while it is written
   if (lane == 0) {
     int c = lastBest + 1;
     for (int i = length - 1; i >= 0; --i) {
-      const uint32_t m = g.node_meta(c - 1);
-      F->corridor[i] = (uint16_t)meta_id(m);
-      c = (int)meta_pidx(m);
+      F->corridor[i] = (uint16_t)link_id(g.link<true>(c - 1));
+      c = (int)state_pidx(g.state<true>(c - 1));
     }
   }
   wave_sync();

@@ -44,4 +44,7 @@ void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,
                           hipStream_t st);
 
+// Wavefronts of the A* kernel that one compute unit holds at once (bounded by their LDS).
+uint32_t geodesic_blocks_per_cu();
+
 }  // namespace bpsx

@@ -396,6 +396,12 @@ __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 // ------------------------------------------------------------------ launch wrappers
 static inline dim3 grid_for(uint32_t n, uint32_t block) { return dim3((n + block - 1) / block); }
 
+uint32_t geodesic_blocks_per_cu() {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_geodesic, 64, 0) != hipSuccess || n < 1) n = 1;
+  return (uint32_t)n;
+}
+
 void launch_geodesic(const NavData& nav, const GeoQuery* queries, const uint32_t* count, uint32_t* head, float* out,
                      GeoSlot* slots, uint32_t num_blocks, uint64_t* counters, hipStream_t st) {
   hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(64), 0, st, nav, queries, count, head, out, slots, counters);
