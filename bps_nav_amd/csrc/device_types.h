@@ -115,13 +115,13 @@ struct NavData {
   const float* episodes;   // [.][10]
 };
 
-// A* node of the per-slot pool (dtNode, DetourNode.h:36-45) as spilled to HBM: 32 bytes.
+// A* node of the per-slot pool (dtNode, DetourNode.h:36-45) as kept in HBM: 32 bytes.
 struct ANode {
   float pos[3];
+  uint32_t state;  // flags (1 open, 2 closed) | 1-based parent node index << 2
   float cost;
   float total;
   uint32_t link;   // polygon index within the scene (bits 0-14) | next node of the hash chain << 16
-  uint32_t state;  // flags (1 open, 2 closed) | 1-based parent node index << 2
   uint32_t pad;
 };
 static_assert(sizeof(ANode) == 32, "ANode");
@@ -131,7 +131,8 @@ struct HeapEntry {
   uint32_t node;
 };
 
-// Spill area of one A* wavefront in HBM: nodes and open-list entries beyond what its LDS holds.
+// HBM slot of one A* wavefront: the node pool (LDS caches its hot part) and the open-list
+// entries beyond what LDS holds.
 struct alignas(128) GeoSlot {
   ANode nodes[kMaxNodes];
   HeapEntry heap_spill[kMaxNodes];

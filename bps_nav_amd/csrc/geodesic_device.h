@@ -3,16 +3,21 @@
 // conventions of the reference, so that the value equals PathFinder::findPath's.
 //
 // Execution model: one wavefront (64 lanes) owns one query at a time and pulls the next from
-// a shared queue when done.  The whole working set of A* lives in LDS: the open list (a binary
-// heap), the hash heads and chains of the node pool, and the first kNodesLds nodes; only
-// nodes beyond that and heap entries beyond kHeapLds spill to a per-wavefront slot in HBM.
-// A query runs the LDS-only instantiation of the loop until its pool or heap could outgrow
-// LDS within one more expansion, then carries on in the spilling instantiation.  Per expanded
-// node the only HBM traffic is the polygon's six 16-byte edge records: lane j of the wavefront
-// handles edge j (node lookup, cost, heuristic); heap updates are then applied in edge order,
-// which is what makes the result identical to the sequential algorithm, ties included.
-// Everything that is the same for all lanes (heap walks, counters, the expanded node) is kept
-// in scalar registers and branches on the scalar unit.
+// a shared queue when done.  The search touches almost only nodes it created recently (the
+// frontier of A* is narrow), so LDS holds what is hot and small and HBM holds the rest:
+//   - the open list (a binary heap) and the hash heads of the node pool,
+//   - for the first kLinksLds nodes the hash chain link + polygon id and the flags + parent,
+//   - the position, cost and total of the kWindow most recently created nodes (slot = index
+//     modulo kWindow); every write of those also goes to the wavefront's slot in HBM, so an
+//     older node is simply read from there.
+// Heap entries beyond kHeapLds and links beyond kLinksLds spill to the same slot.  A query
+// runs the instantiation of the loop without link/heap spill code until one more expansion
+// could outgrow either, then carries on in the spilling instantiation.  Per expanded node the
+// regular HBM traffic is the polygon's six 16-byte edge records (lane j of the wavefront
+// handles edge j: node lookup, cost, heuristic) plus the write-through of updated nodes; heap
+// updates are applied in edge order, which is what makes the result identical to the
+// sequential algorithm, ties included.  Everything that is the same for all lanes (heap walks,
+// counters, the expanded node) is kept in scalar registers and branches on the scalar unit.
 //
 // Reference semantics followed: DetourNavMeshQuery.cpp:945-1178 (findPath, getPathToNode),
 // :1661-1696, 1765-1994 (appendVertex, findStraightPath), :2279-2381 (getPortalPoints,
@@ -28,15 +33,20 @@ namespace bpsx {
 #define PHASE_MARK(k) do { } while (0)
 #endif
 
-#ifndef BPSX_NODES_LDS
-#define BPSX_NODES_LDS 512
+#ifndef BPSX_LINKS_LDS
+#define BPSX_LINKS_LDS 768
 #endif
 #ifndef BPSX_HEAP_LDS
-#define BPSX_HEAP_LDS 256
+#define BPSX_HEAP_LDS 128
 #endif
-constexpr int kNodesLds = BPSX_NODES_LDS;   // nodes kept in LDS per query
-constexpr int kHeapLds = BPSX_HEAP_LDS;     // open-list entries kept in LDS per query
+#ifndef BPSX_WINDOW
+#define BPSX_WINDOW 128
+#endif
+constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link and state words are kept in LDS
+constexpr int kHeapLds = BPSX_HEAP_LDS;     // open-list entries kept in LDS
+constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
 constexpr int kHashSize = 512;
+static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
 
 BPSX_DEV void wave_sync() {
   // All lanes belong to one wavefront: LDS and memory operations issue in program order, so
@@ -51,20 +61,27 @@ BPSX_DEV int lane_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane)
 
 // LDS of one wavefront.
 struct GeoLds {
-  float n_total[kNodesLds];
-  float n_cost[kNodesLds];
-  float n_pos[3][kNodesLds];
-  uint32_t n_link[kNodesLds];      // polygon index (bits 0-14) | next node of the hash chain << 16
-  uint16_t n_state[kNodesLds];     // flags (1 open, 2 closed) | 1-based parent node index << 2
   uint16_t first[kHashSize];
   HeapEntry heap[kHeapLds];
+  uint32_t n_link[kLinksLds];      // polygon index (bits 0-14) | next node of the hash chain << 16
+  uint16_t n_state[kLinksLds];     // flags (1 open, 2 closed) | 1-based parent node index << 2
+  float w_total[kWindow];
+  float w_cost[kWindow];
+  float w_pos[3][kWindow];
 };
-// After A* the node arrays are dead; the funnel reuses them for the corridor and its portals.
+// After A* its LDS is dead; the funnel reuses it for the corridor and its portals.  The
+// corridor is written while the nodes' links and parent indices are still being read: it lies
+// over the hash heads, which are no longer needed by then.
 struct FunnelLds {
-  float portals[kMaxPath][6];
   uint16_t corridor[kMaxPath];
+  uint16_t pad[kHashSize - kMaxPath];
+  float portals[kMaxPath][6];
 };
-static_assert(sizeof(FunnelLds) <= offsetof(GeoLds, n_link), "funnel scratch must stay clear of the node links");
+static_assert(offsetof(FunnelLds, portals) == offsetof(GeoLds, heap), "corridor must overlay the hash heads only");
+union GeoShared {
+  GeoLds a;
+  FunnelLds f;
+};
 
 constexpr uint32_t kChainEnd = 0xffffu;
 BPSX_DEV uint32_t link_id(uint32_t l) { return l & 0x7fffu; }
@@ -72,8 +89,8 @@ BPSX_DEV uint32_t link_next(uint32_t l) { return l >> 16; }
 BPSX_DEV uint32_t state_flags(uint32_t s) { return s & 3u; }
 BPSX_DEV uint32_t state_pidx(uint32_t s) { return s >> 2; }
 
-// Accessors take the instantiation's spill switch S: with S false every index is known to be
-// inside LDS and no address-space branch is generated.
+// Accessors take the instantiation's spill switch S: with S false every node index is below
+// kLinksLds and every heap index below kHeapLds, and no address-space branch is generated.
 struct GeoWave {
   GeoLds* L;
   GeoSlot* ws;
@@ -82,16 +99,18 @@ struct GeoWave {
   int nodeCount;
 
   // ---------------------------------------------------------------- node pool
-  template <bool S> BPSX_DEV uint32_t link(int i) const { return (!S || i < kNodesLds) ? L->n_link[i] : ws->nodes[i].link; }
+  template <bool S> BPSX_DEV uint32_t link(int i) const { return (!S || i < kLinksLds) ? L->n_link[i] : ws->nodes[i].link; }
   template <bool S> BPSX_DEV void set_link(int i, uint32_t v) const {
-    if (!S || i < kNodesLds) L->n_link[i] = v;
+    if (!S || i < kLinksLds) L->n_link[i] = v;
     else ws->nodes[i].link = v;
   }
-  template <bool S> BPSX_DEV uint32_t state(int i) const { return (!S || i < kNodesLds) ? (uint32_t)L->n_state[i] : ws->nodes[i].state; }
+  template <bool S> BPSX_DEV uint32_t state(int i) const { return (!S || i < kLinksLds) ? (uint32_t)L->n_state[i] : ws->nodes[i].state; }
   template <bool S> BPSX_DEV void set_state(int i, uint32_t v) const {
-    if (!S || i < kNodesLds) L->n_state[i] = (uint16_t)v;
+    if (!S || i < kLinksLds) L->n_state[i] = (uint16_t)v;
     else ws->nodes[i].state = v;
   }
+  // node i still has its position/cost/total in LDS
+  BPSX_DEV bool in_window(int i) const { return i >= nodeCount - kWindow; }
   static BPSX_DEV uint32_t hash(uint32_t ip) { return (__umul24(ip, 0x9e3779u) >> 9) & (kHashSize - 1); }
   BPSX_DEV void clear() {
     for (int i = lane; i < kHashSize; i += 64) L->first[i] = (uint16_t)kChainEnd;
@@ -196,21 +215,19 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const float H_SCALE = 0.999f;
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
   while (g.heapSize > 0) {
-    if (!S && (g.nodeCount > kNodesLds - kNvp || g.heapSize > kHeapLds - kNvp)) return kAstarGrow;
+    if (!S && (g.nodeCount > kLinksLds - kNvp || g.heapSize > kHeapLds - kNvp)) return kAstarGrow;
     // the node about to be popped is the root: fetch its edges while the heap is repaired
     const int bi = uniform_i((int)L->heap[0].node);
     float b0, b1, b2, bcost;
-    uint32_t bestIp, pidx;
-    if (!S || bi < kNodesLds) {
-      b0 = L->n_pos[0][bi]; b1 = L->n_pos[1][bi]; b2 = L->n_pos[2][bi]; bcost = L->n_cost[bi];
-      bestIp = link_id((uint32_t)uniform_i((int)L->n_link[bi]));
-      pidx = state_pidx((uint32_t)uniform_i((int)L->n_state[bi]));
+    if (g.in_window(bi)) {
+      const int w = bi & (kWindow - 1);
+      b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
     } else {
       const ANode& n = g.ws->nodes[bi];
       b0 = n.pos[0]; b1 = n.pos[1]; b2 = n.pos[2]; bcost = n.cost;
-      bestIp = link_id((uint32_t)uniform_i((int)n.link));
-      pidx = state_pidx((uint32_t)uniform_i((int)n.state));
     }
+    const uint32_t bestIp = link_id((uint32_t)uniform_i((int)g.link<S>(bi)));
+    const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)g.state<S>(bi)));
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
     if (lane < kNvp) {
@@ -273,13 +290,15 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (nb != kNoNb) {
       float p0 = m0, p1 = m1, p2 = m2, oldTotal = 0;
       uint32_t fl = 0;
+      const bool inw = g.in_window(ni);   // new nodes always are
+      const int w = ni & (kWindow - 1);
+      ANode& hn = g.ws->nodes[ni];
       if (!isNew) {
-        if (!S || ni < kNodesLds) {
-          p0 = L->n_pos[0][ni]; p1 = L->n_pos[1][ni]; p2 = L->n_pos[2][ni];
-          oldTotal = L->n_total[ni]; fl = state_flags(L->n_state[ni]);
+        fl = state_flags(g.state<S>(ni));
+        if (inw) {
+          p0 = L->w_pos[0][w]; p1 = L->w_pos[1][w]; p2 = L->w_pos[2][w]; oldTotal = L->w_total[w];
         } else {
-          const ANode& n = g.ws->nodes[ni];
-          p0 = n.pos[0]; p1 = n.pos[1]; p2 = n.pos[2]; oldTotal = n.total; fl = state_flags(n.state);
+          p0 = hn.pos[0]; p1 = hn.pos[1]; p2 = hn.pos[2]; oldTotal = hn.total;
         }
       }
       const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
@@ -299,15 +318,13 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       if (!worse) {
         update = true;
         wasOpen = (fl & 1u) != 0;
-        const uint32_t ns = 1u | ((uint32_t)(bi + 1) << 2);   // open, parent = expanded node
-        if (!S || ni < kNodesLds) {
-          if (isNew) { L->n_pos[0][ni] = p0; L->n_pos[1][ni] = p1; L->n_pos[2][ni] = p2; }
-          L->n_cost[ni] = cost; L->n_total[ni] = total; L->n_state[ni] = (uint16_t)ns;
-        } else {
-          ANode& n = g.ws->nodes[ni];
-          if (isNew) { n.pos[0] = p0; n.pos[1] = p1; n.pos[2] = p2; }
-          n.cost = cost; n.total = total; n.state = ns;
+        g.set_state<S>(ni, 1u | ((uint32_t)(bi + 1) << 2));   // open, parent = expanded node
+        if (inw) {
+          if (isNew) { L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2; }
+          L->w_cost[w] = cost; L->w_total[w] = total;
         }
+        if (isNew) { hn.pos[0] = p0; hn.pos[1] = p1; hn.pos[2] = p2; }
+        hn.cost = cost; hn.total = total;
       }
     }
     wave_sync();
@@ -355,8 +372,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     g.nodeCount = 1;
     if (lane == 0) {
       GeoLds* L = g.L;
-      L->n_pos[0][0] = startPos[0]; L->n_pos[1][0] = startPos[1]; L->n_pos[2][0] = startPos[2];
-      L->n_cost[0] = 0; L->n_total[0] = total;
+      ANode& hn = g.ws->nodes[0];
+      for (int k = 0; k < 3; ++k) { L->w_pos[k][0] = startPos[k]; hn.pos[k] = startPos[k]; }
+      L->w_cost[0] = 0; L->w_total[0] = total;
+      hn.cost = 0; hn.total = total;
       L->n_state[0] = 1;   // open, no parent
       L->n_link[0] = startIp | (kChainEnd << 16);
       L->first[GeoWave::hash(startIp)] = 0;
@@ -524,7 +543,7 @@ BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q,
   if (sIp == kInvalidPoly || eIp == kInvalidPoly) return INF;
   if (nav.polys[s.poly_base + sIp].island != nav.polys[s.poly_base + eIp].island) return INF;
   if (!finite3(q.a[0], q.a[1], q.a[2]) || !finite3(q.b[0], q.b[1], q.b[2])) return INF;
-  FunnelLds* F = reinterpret_cast<FunnelLds*>(g.L);
+  FunnelLds* F = &reinterpret_cast<GeoShared*>(g.L)->f;
 #ifdef BPSX_PHASE_TIMING
   const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops, phase_acc);
   unsigned long long phase_t0 = __builtin_readcyclecounter();

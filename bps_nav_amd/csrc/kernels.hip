@@ -310,10 +310,10 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
 __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries,
                                                  const uint32_t* __restrict__ count, uint32_t* head, float* out,
                                                  GeoSlot* slots, uint64_t* counters) {
-  __shared__ GeoLds lds;
+  __shared__ GeoShared lds;
   GeoWave g;
   g.lane = (int)threadIdx.x;
-  g.L = &lds;
+  g.L = &lds.a;
   g.ws = &slots[blockIdx.x];
   g.heapSize = 0;
   g.nodeCount = 0;
