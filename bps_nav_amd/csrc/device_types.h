@@ -116,11 +116,11 @@ struct NavData {
 };
 
 // A* node of the per-slot pool (dtNode, DetourNode.h:36-45) as kept in HBM: 32 bytes.
-struct ANode {
+struct alignas(16) ANode {
   float pos[3];
-  uint32_t state;  // flags (1 open, 2 closed) | 1-based parent node index << 2
   float cost;
   float total;
+  uint32_t state;  // flags (1 open, 2 closed) | 1-based parent node index << 2
   uint32_t link;   // polygon index within the scene (bits 0-14) | next node of the hash chain << 16
   uint32_t pad;
 };

@@ -5,14 +5,16 @@
 // Execution model: one wavefront (64 lanes) owns one query at a time and pulls the next from
 // a shared queue when done.  The search touches almost only nodes it created recently (the
 // frontier of A* is narrow), so LDS holds what is hot and small and HBM holds the rest:
-//   - the open list (a binary heap) and the hash heads of the node pool,
+//   - the open list, a binary heap, in registers while it has fewer than 128 entries (entry q
+//     in lane q mod 64), then in LDS,
+//   - the hash heads of the node pool,
 //   - for the first kLinksLds nodes the hash chain link + polygon id and the flags + parent,
 //   - the position, cost and total of the kWindow most recently created nodes (slot = index
 //     modulo kWindow); every write of those also goes to the wavefront's slot in HBM, so an
 //     older node is simply read from there.
 // Heap entries beyond kHeapLds and links beyond kLinksLds spill to the same slot.  A query
-// runs the instantiation of the loop without link/heap spill code until one more expansion
-// could outgrow either, then carries on in the spilling instantiation.  Per expanded node the
+// runs the instantiation of the loop without spill code until one more expansion could
+// outgrow the links in LDS or the register heap, then carries on in a spilling instantiation.  Per expanded node the
 // regular HBM traffic is the polygon's six 16-byte edge records (lane j of the wavefront
 // handles edge j: node lookup, cost, heuristic) plus the write-through of updated nodes; heap
 // updates are applied in edge order, which is what makes the result identical to the
@@ -27,7 +29,9 @@
 
 namespace bpsx {
 
-#ifdef BPSX_PHASE_TIMING
+#ifdef BPSX_ASM_MARKS
+#define PHASE_MARK(k) asm volatile("; PHASE_MARK " #k)
+#elif defined(BPSX_PHASE_TIMING)
 #define PHASE_MARK(k) do { const unsigned long long now_ = __builtin_readcyclecounter(); phase_acc[k] += now_ - phase_t0; phase_t0 = now_; } while (0)
 #else
 #define PHASE_MARK(k) do { } while (0)
@@ -58,6 +62,14 @@ BPSX_DEV int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
 BPSX_DEV float uniform_f(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 BPSX_DEV float lane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
 BPSX_DEV int lane_i(int v, int lane) { return __builtin_amdgcn_readlane(v, lane); }
+BPSX_DEV uint32_t rlane(uint32_t v, int lane) { return (uint32_t)__builtin_amdgcn_readlane((int)v, lane); }
+// old with lane `lane` replaced by v (v and lane uniform).  The lane select travels in M0:
+// gfx9 encodings take at most one general scalar register per vector instruction.
+BPSX_DEV uint32_t wlane(uint32_t old, uint32_t v, int lane) {
+  const int sv = __builtin_amdgcn_readfirstlane((int)v), sl = __builtin_amdgcn_readfirstlane(lane);
+  asm("s_mov_b32 m0, %2\n\tv_writelane_b32 %0, %1, m0" : "+v"(old) : "s"(sv), "s"(sl) : "m0");
+  return old;
+}
 
 // LDS of one wavefront.
 struct GeoLds {
@@ -195,16 +207,93 @@ struct GeoWave {
   }
 };
 
+// The open list in registers.  Heap position q (1-based, root = 1; the reference's index + 1)
+// lives in lane q & 63 of the first register pair (q < 64) or of the second (64 <= q < 128).
+// Totals are kept as bit patterns and compared as unsigned integers on the scalar unit: they
+// are sums of distances, never negative and never NaN, and for such floats the integer order
+// of the bits is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
+constexpr int kRegHeap = 127;
+static_assert(kHeapLds > kRegHeap, "the register heap must fit the LDS heap it is moved to");
+struct RegHeap {
+  uint32_t t0, t1;   // total bits
+  uint32_t n0, n1;   // node index
+  int size;
+
+  BPSX_DEV uint32_t T(int q) const { return q < 64 ? rlane(t0, q) : rlane(t1, q & 63); }
+  BPSX_DEV uint32_t N(int q) const { return q < 64 ? rlane(n0, q) : rlane(n1, q & 63); }
+  BPSX_DEV void set(int q, uint32_t t, uint32_t n) {
+    if (q < 64) { t0 = wlane(t0, t, q); n0 = wlane(n0, n, q); }
+    else { t1 = wlane(t1, t, q & 63); n1 = wlane(n1, n, q & 63); }
+  }
+  BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n) {
+    while (q > 1) {
+      const int p = q >> 1;
+      const uint32_t pt = T(p);
+      if (!(pt > t)) break;
+      set(q, pt, N(p));
+      q = p;
+    }
+    set(q, t, n);
+  }
+  BPSX_DEV void push(uint32_t t, uint32_t n) {
+    size++;
+    bubble_up(size, t, n);
+  }
+  BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
+    int q = 0;
+    unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);
+    if (m) q = __ffsll((long long)m) - 1;
+    else {
+      m = __ballot(64 + lane <= size && n1 == n);
+      if (m) q = 64 + __ffsll((long long)m) - 1;
+    }
+    if (q) bubble_up(q, t, n);
+  }
+  // pop after the caller has taken the root: the hole moves down along the smaller children
+  // while they are not greater than the former last entry, which then fills it (the
+  // reference moves the hole to a leaf first and bubbles the entry back up: same result).
+  // Positions past the end hold kEmpty, greater than any total, so the walk needs no bounds.
+  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
+  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
+  BPSX_DEV void pop() {
+    const int last = size;
+    size--;
+    uint32_t lt, ln;
+    if (last < 64) { lt = rlane(t0, last); ln = rlane(n0, last); t0 = wlane(t0, kEmpty, last); }
+    else { lt = rlane(t1, last & 63); ln = rlane(n1, last & 63); t1 = wlane(t1, kEmpty, last & 63); }
+    if (size == 0) return;
+    uint32_t q = 1;
+#pragma unroll
+    for (int lvl = 0; lvl < 6; ++lvl) {   // children of levels 0-4 are in the first register pair
+      uint32_t c = 2 * q;
+      const uint32_t tl = lvl < 5 ? rlane(t0, (int)c) : rlane(t1, (int)(c & 63));
+      const uint32_t tr = lvl < 5 ? rlane(t0, (int)c + 1) : rlane(t1, (int)((c + 1) & 63));
+      // keys are below 2^31: the sign of the difference is the comparison, on the scalar unit
+      const uint32_t right = (tr - tl) >> 31;   // 1 when the right child is smaller
+      c += right;
+      const uint32_t tc = right ? tr : tl;
+      if ((lt - tc) >> 31) break;               // child greater than the entry: it stays below
+      const uint32_t nc = lvl < 5 ? rlane(n0, (int)c) : rlane(n1, (int)(c & 63));
+      t0 = wlane(t0, tc, (int)q);
+      n0 = wlane(n0, nc, (int)q);
+      q = c;
+    }
+    set((int)q, lt, ln);
+  }
+};
+
 struct AstarState {
   int lastBest;
   float lastBestCost;
   bool outOfNodes;
+  RegHeap rh;
 };
-enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrow = 2 };
+enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
 
-// The expansion loop of findPath. S = false: all nodes and heap entries are in LDS; returns
-// kAstarGrow before an expansion that could need more than LDS holds.
-template <bool S>
+// The expansion loop of findPath.  M = 0: open list in registers, all links in LDS; M = 1: open
+// list in registers, links may spill; M = 2: open list in LDS/HBM, links may spill.  Returns
+// kAstarGrow* before an expansion that could outgrow what its mode holds.
+template <int M>
 BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
 #ifdef BPSX_PHASE_TIMING
                               , unsigned long long* phase_acc, unsigned long long& phase_t0
@@ -214,17 +303,21 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
   GeoLds* L = g.L;
   const float H_SCALE = 0.999f;
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
-  while (g.heapSize > 0) {
-    if (!S && (g.nodeCount > kLinksLds - kNvp || g.heapSize > kHeapLds - kNvp)) return kAstarGrow;
+  constexpr bool S = M >= 1;    // links and states may be in HBM
+  constexpr bool SH = M == 2;   // open list in LDS/HBM
+  RegHeap& rh = st.rh;
+  while ((SH ? g.heapSize : rh.size) > 0) {
+    if (M == 0 && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
+    if (!SH && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
     // the node about to be popped is the root: fetch its edges while the heap is repaired
-    const int bi = uniform_i((int)L->heap[0].node);
+    const int bi = SH ? uniform_i((int)L->heap[0].node) : (int)rlane(rh.n0, 1);
     float b0, b1, b2, bcost;
     if (g.in_window(bi)) {
       const int w = bi & (kWindow - 1);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
     } else {
-      const ANode& n = g.ws->nodes[bi];
-      b0 = n.pos[0]; b1 = n.pos[1]; b2 = n.pos[2]; bcost = n.cost;
+      const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
+      b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
     }
     const uint32_t bestIp = link_id((uint32_t)uniform_i((int)g.link<S>(bi)));
     const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)g.state<S>(bi)));
@@ -235,21 +328,12 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
     PHASE_MARK(0);
-    g.pop<S>();
+    if (SH) g.pop<true>();
+    else rh.pop();
     PHASE_MARK(1);
     g.set_state<S>(bi, 2u | (pidx << 2));   // open -> closed
     if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
     (*pops)++;
-    // a polygon reached through two edges of the same expansion: the second visit never
-    // changes the node (same position, same cost), so only the first edge counts
-    {
-      const uint32_t orig = nb;
-#pragma unroll
-      for (int k = 0; k < kNvp - 1; ++k) {
-        const uint32_t other = (uint32_t)lane_i((int)orig, k);
-        if (lane > k && other == orig) nb = kNoNb;
-      }
-    }
     PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
     int ni = -1;
@@ -298,7 +382,9 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         if (inw) {
           p0 = L->w_pos[0][w]; p1 = L->w_pos[1][w]; p2 = L->w_pos[2][w]; oldTotal = L->w_total[w];
         } else {
-          p0 = hn.pos[0]; p1 = hn.pos[1]; p2 = hn.pos[2]; oldTotal = hn.total;
+          const float4 pc = *reinterpret_cast<const float4*>(hn.pos);   // pos, cost
+          const float2 ts = *reinterpret_cast<const float2*>(&hn.total);  // total, state
+          p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = ts.x;
         }
       }
       const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
@@ -323,23 +409,30 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
           if (isNew) { L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2; }
           L->w_cost[w] = cost; L->w_total[w] = total;
         }
-        if (isNew) { hn.pos[0] = p0; hn.pos[1] = p1; hn.pos[2] = p2; }
-        hn.cost = cost; hn.total = total;
+        if (isNew) *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
+        else hn.cost = cost;
+        hn.total = total;
       }
     }
     wave_sync();
     PHASE_MARK(5);
     // ---- ordered phase: heap and "nearest so far" updates in edge order
     unsigned long long upd = __ballot(update);
+    const unsigned long long openMask = __ballot(update && wasOpen);
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
       const int node = lane_i(ni, src);
       const float t = lane_f(total, src);
       const float h = lane_f(heuristic, src);
-      const bool open = lane_i(wasOpen ? 1 : 0, src) != 0;
-      if (open) g.modify<S>(node, t);
-      else g.push<S>(t, node);
+      const bool open = (openMask >> src) & 1ull;
+      if (SH) {
+        if (open) g.modify<true>(node, t);
+        else g.push<true>(t, node);
+      } else {
+        if (open) rh.modify((uint32_t)node, __float_as_uint(t), lane);
+        else rh.push(__float_as_uint(t), (uint32_t)node);
+      }
       if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = node; }
     }
     PHASE_MARK(6);
@@ -381,19 +474,30 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       L->first[GeoWave::hash(startIp)] = 0;
     }
     wave_sync();
-    g.push<false>(total, 0);
+    st.rh.init();
+    st.rh.push(__float_as_uint(total), 0u);
     st.lastBest = 0;
     st.lastBestCost = total;
     st.outOfNodes = false;
   }
   const AEdge* edges = nav.aedges + (size_t)s.poly_base * kNvp;
 #ifdef BPSX_PHASE_TIMING
-  AstarExit ex = astar_loop<false>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0);
-  if (ex == kAstarGrow) ex = astar_loop<true>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0);
+#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0)
 #else
-  AstarExit ex = astar_loop<false>(g, st, edges, endIp, endPos, pops);
-  if (ex == kAstarGrow) ex = astar_loop<true>(g, st, edges, endIp, endPos, pops);
+#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
 #endif
+  AstarExit ex = ASTAR_RUN(0);
+  if (ex == kAstarGrowLinks) ex = ASTAR_RUN(1);
+  if (ex == kAstarGrowHeap) {
+    // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
+    const RegHeap& rh = st.rh;
+    if (lane >= 1 && lane <= rh.size) g.L->heap[lane - 1] = HeapEntry{__uint_as_float(rh.t0), rh.n0};
+    if (64 + lane <= rh.size) g.L->heap[63 + lane] = HeapEntry{__uint_as_float(rh.t1), rh.n1};
+    g.heapSize = rh.size;
+    wave_sync();
+    ex = ASTAR_RUN(2);
+  }
+#undef ASTAR_RUN
   (void)ex;
   const int lastBest = st.lastBest;
   // getPathToNode

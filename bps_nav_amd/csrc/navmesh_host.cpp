@@ -155,6 +155,10 @@ int parse_navmesh(const uint8_t* b, size_t n, HostScene* out) {
       const float* rt = r.v[(k + 1) % r.nv];
       for (int c = 0; c < 3; ++c) e.mid[c] = (l[c] + rt[c]) * 0.5f;
       e.nb = r.walk[k] ? (uint32_t)(r.walk[k] - 1) : kNoNb;
+      // a polygon behind two edges: expanding through the second never changes its node (same
+      // position, not a lower cost), so only the first edge leads there
+      for (int j = 0; j < k; ++j)
+        if (r.walk[j] == r.walk[k]) e.nb = kNoNb;
     }
   }
   // connected components: polygons are seeded in index order, the seed is not filter-checked,
