@@ -58,6 +58,9 @@ BPSX_DEV void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   __builtin_amdgcn_wave_barrier();
 }
+// Keeps the compiler from folding an LDS access and an HBM access of two branches into one
+// generic-address access (which would wait on both memory counters and on pending stores).
+#define BPSX_KEEP_APART() asm volatile("")
 BPSX_DEV int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
 BPSX_DEV float uniform_f(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 BPSX_DEV float lane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
@@ -111,15 +114,27 @@ struct GeoWave {
   int nodeCount;
 
   // ---------------------------------------------------------------- node pool
-  template <bool S> BPSX_DEV uint32_t link(int i) const { return (!S || i < kLinksLds) ? L->n_link[i] : ws->nodes[i].link; }
+  template <bool S> BPSX_DEV uint32_t link(int i) const {
+    if (!S || i < kLinksLds) return L->n_link[i];
+    BPSX_KEEP_APART();
+    const uint32_t v = ws->nodes[i].link;
+    BPSX_KEEP_APART();
+    return v;
+  }
   template <bool S> BPSX_DEV void set_link(int i, uint32_t v) const {
     if (!S || i < kLinksLds) L->n_link[i] = v;
-    else ws->nodes[i].link = v;
+    else { BPSX_KEEP_APART(); ws->nodes[i].link = v; BPSX_KEEP_APART(); }
   }
-  template <bool S> BPSX_DEV uint32_t state(int i) const { return (!S || i < kLinksLds) ? (uint32_t)L->n_state[i] : ws->nodes[i].state; }
+  template <bool S> BPSX_DEV uint32_t state(int i) const {
+    if (!S || i < kLinksLds) return (uint32_t)L->n_state[i];
+    BPSX_KEEP_APART();
+    const uint32_t v = ws->nodes[i].state;
+    BPSX_KEEP_APART();
+    return v;
+  }
   template <bool S> BPSX_DEV void set_state(int i, uint32_t v) const {
     if (!S || i < kLinksLds) L->n_state[i] = (uint16_t)v;
-    else ws->nodes[i].state = v;
+    else { BPSX_KEEP_APART(); ws->nodes[i].state = v; BPSX_KEEP_APART(); }
   }
   // node i still has its position/cost/total in LDS
   BPSX_DEV bool in_window(int i) const { return i >= nodeCount - kWindow; }
@@ -144,11 +159,17 @@ struct GeoWave {
   // The heap is walked with wave-uniform indices: every lane issues the same LDS access and the
   // values are moved to scalar registers, so the loops below branch on the scalar unit and cost
   // a handful of vector instructions per level.
-  template <bool S> BPSX_DEV HeapEntry hget(int i) const { return (!S || i < kHeapLds) ? L->heap[i] : ws->heap_spill[i]; }
+  template <bool S> BPSX_DEV HeapEntry hget(int i) const {
+    if (!S || i < kHeapLds) return L->heap[i];
+    BPSX_KEEP_APART();
+    const HeapEntry e = ws->heap_spill[i];
+    BPSX_KEEP_APART();
+    return e;
+  }
   template <bool S> BPSX_DEV void hset(int i, float t, int n) const {
     const HeapEntry e{t, (uint32_t)n};
     if (!S || i < kHeapLds) L->heap[i] = e;   // all lanes store the same value to the same address
-    else if (lane == 0) ws->heap_spill[i] = e;
+    else if (lane == 0) { BPSX_KEEP_APART(); ws->heap_spill[i] = e; BPSX_KEEP_APART(); }
   }
   // dtNodeQueue::bubbleUp from index i with entry (t, n)
   template <bool S> BPSX_DEV void bubble_up(int i, float t, int n) const {
@@ -316,8 +337,10 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const int w = bi & (kWindow - 1);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
     } else {
+      BPSX_KEEP_APART();
       const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
       b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
+      BPSX_KEEP_APART();
     }
     const uint32_t bestIp = link_id((uint32_t)uniform_i((int)g.link<S>(bi)));
     const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)g.state<S>(bi)));
@@ -382,9 +405,11 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         if (inw) {
           p0 = L->w_pos[0][w]; p1 = L->w_pos[1][w]; p2 = L->w_pos[2][w]; oldTotal = L->w_total[w];
         } else {
+          BPSX_KEEP_APART();
           const float4 pc = *reinterpret_cast<const float4*>(hn.pos);   // pos, cost
           const float2 ts = *reinterpret_cast<const float2*>(&hn.total);  // total, state
           p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = ts.x;
+          BPSX_KEEP_APART();
         }
       }
       const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
@@ -480,7 +505,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.lastBestCost = total;
     st.outOfNodes = false;
   }
-  const AEdge* edges = nav.aedges + (size_t)s.poly_base * kNvp;
+  const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kNvp;
 #ifdef BPSX_PHASE_TIMING
 #define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0)
 #else
