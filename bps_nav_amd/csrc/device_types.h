@@ -148,7 +148,8 @@ struct GeoQuery {
 };
 
 enum Counter {
-  kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands
+  kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,
+  kCntLinkSpills = 16, kCntHeapSpills = 17   // 8..15: phase cycles of the diagnostic build
 };
 
 }  // namespace bpsx

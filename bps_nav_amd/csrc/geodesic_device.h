@@ -112,6 +112,7 @@ struct GeoWave {
   int lane;
   int heapSize;
   int nodeCount;
+  uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
 
   // ---------------------------------------------------------------- node pool
   template <bool S> BPSX_DEV uint32_t link(int i) const {
@@ -512,8 +513,9 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
 #endif
   AstarExit ex = ASTAR_RUN(0);
-  if (ex == kAstarGrowLinks) ex = ASTAR_RUN(1);
+  if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
   if (ex == kAstarGrowHeap) {
+    g.heapSpills++;
     // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
     const RegHeap& rh = st.rh;
     if (lane >= 1 && lane <= rh.size) g.L->heap[lane - 1] = HeapEntry{__uint_as_float(rh.t0), rh.n0};

@@ -317,6 +317,7 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
   g.ws = &slots[blockIdx.x];
   g.heapSize = 0;
   g.nodeCount = 0;
+  g.linkSpills = g.heapSpills = 0;
   const uint32_t nq = *count;
   uint32_t pops = 0, corridor = 0, done = 0;
 #ifdef BPSX_PHASE_TIMING
@@ -341,6 +342,8 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
     atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)done);
     atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)pops);
     atomicAdd((unsigned long long*)&counters[kCntCorridor], (unsigned long long)corridor);
+    if (g.linkSpills) atomicAdd((unsigned long long*)&counters[kCntLinkSpills], (unsigned long long)g.linkSpills);
+    if (g.heapSpills) atomicAdd((unsigned long long*)&counters[kCntHeapSpills], (unsigned long long)g.heapSpills);
 #ifdef BPSX_PHASE_TIMING
     for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], phase_acc[k]);
 #endif

@@ -60,11 +60,45 @@ def test_batched_queries_match_oracle(oracle, torch_cuda, config):
     gg = gen.geodesic(0, a, ar, b, br)
     assert np.array_equal(common.bits(go), common.bits(gg)), \
         f"{(common.bits(go) != common.bits(gg)).sum()} of {m} geodesics differ"
+    if config == 4:  # maze-wide pairs: searches that outgrow the node links kept in LDS
+        assert gen.counters()["geo_link_spills"] > 20
     # invalid refs and coincident points
     gz = gen.geodesic(0, a[:4], ar[:4], a[:4], ar[:4])
     assert (gz == 0).all()
     gi = gen.geodesic(0, a[:4], np.zeros(4, np.uint32), b[:4], br[:4])
     assert np.isinf(gi).all()
+    gen.close()
+
+
+def test_open_hall_queries_match_oracle(oracle, torch_cuda):
+    """A hall without obstacles: A* spreads over a wide front, so the open list outgrows the
+    kernel's register heap, the node links outgrow LDS and long queries exhaust Detour's
+    2048-node pool.  Every continuation path of the kernel must still equal the oracle."""
+    from bps_nav_amd import scenes
+    from oracle import bpo
+    print("case: open hall (spill paths of the A* kernel)", flush=True)
+    blob = scenes.gen_scene(scenes.BOX_ROOM, 4242, cell=5, size_x=30.0, size_z=30.0, num_boxes=0, tri_frac=0.2,
+                            hex_frac=0.1)
+    nav = bpo.Nav(oracle, blob)
+    gen = make_gen([(blob, np.zeros((1, 10), np.float32))], 1)
+    pts = scenes.sample_points(blob, 9, 1600)
+    x, r = nav.snap(pts)
+    assert (r != 0).all()
+    m = len(x) // 2
+    a, ar, b, br = x[:m], r[:m], x[m:], r[m:]
+    # mix of ranges: short hops, mid-range (large open list, path found) and far (pool exhausted)
+    k = m // 2
+    b[:k] = a[:k] + (b[:k] - a[:k]) * np.linspace(0.02, 0.5, k, dtype=np.float32)[:, None]
+    b, br = nav.snap(b)
+    c0 = gen.counters()
+    go = nav.geodesic(a, ar, b, br)
+    gg = gen.geodesic(0, a, ar, b, br)
+    c1 = gen.counters()
+    assert np.array_equal(common.bits(go), common.bits(gg)), \
+        f"{(common.bits(go) != common.bits(gg)).sum()} of {m} geodesics differ"
+    assert np.isinf(go).any() and np.isfinite(go).sum() > m // 3
+    assert c1["geo_link_spills"] - c0["geo_link_spills"] > 0, "link spill path not exercised"
+    assert c1["geo_heap_spills"] - c0["geo_heap_spills"] > 20, "heap spill path not exercised"
     gen.close()
 
 
