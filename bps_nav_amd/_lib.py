@@ -13,12 +13,12 @@ LIB_PATH = os.environ.get("BPSX_LIBRARY") or os.path.join(_HERE, "libbpsx.so")
 class Config(C.Structure):
     _fields_ = [("num_environments", C.c_uint32), ("num_active_scenes", C.c_uint32),
                 ("double_buffered", C.c_uint32), ("reset_mode", C.c_uint32), ("seed", C.c_uint64),
-                ("gpu_id", C.c_int32), ("max_steps", C.c_uint32)]
+                ("gpu_id", C.c_int32), ("max_steps", C.c_uint32), ("task", C.c_uint32)]
 
 
 class Outputs(C.Structure):
     _fields_ = [("rewards", C.c_void_p), ("masks", C.c_void_p), ("infos", C.c_void_p),
-                ("polars", C.c_void_p), ("n", C.c_uint32)]
+                ("polars", C.c_void_p), ("n", C.c_uint32), ("info_width", C.c_uint32)]
 
 
 class State(C.Structure):

@@ -18,19 +18,21 @@ INFO_FIELDS = ("success", "spl", "distanceToGoal")  # struct dtype, simulator.cp
 
 
 class _InfoDType:
-    names = INFO_FIELDS
+    def __init__(self, names):
+        self.names = names
 
 
 class InfoView:
     """What get_infos returns: indexable by field name like the reference's structured numpy
     array (env_utils.py:106-110), each field a strided view f32[n] of the device tensor."""
-    dtype = _InfoDType
 
-    def __init__(self, packed):
-        self.packed = packed  # f32[n,3]
+    def __init__(self, packed, fields=INFO_FIELDS):
+        self.packed = packed  # f32[n, len(fields)]
+        self.fields = fields
+        self.dtype = _InfoDType(fields)
 
     def __getitem__(self, key):
-        return self.packed[:, INFO_FIELDS.index(key)]
+        return self.packed[:, self.fields.index(key)]
 
 
 def load_dataset(dataset_path, asset_path):
@@ -66,6 +68,8 @@ class PointNavRolloutGenerator:
     (simulator.cpp:1791-1809).  Renderer arguments are accepted and ignored; `scenes`
     (keyword) supplies in-memory [(navmesh_bytes, episodes f32[E,10])] instead of a dataset
     directory.  Getters return torch tensors that alias the simulator's device buffers."""
+    TASK = 0                      # BPSX_TASK_POINTNAV
+    INFO_FIELDS = INFO_FIELDS     # PointNav::Simulator::StepInfo (simulator.cpp:1814-1815)
 
     def __init__(self, dataset_path, asset_path, num_environments, num_active_scenes, num_workers=-1, gpu_id=0,
                  render_resolution=(64, 64), color=False, depth=False, double_buffered=False, seed=0,
@@ -83,7 +87,7 @@ class PointNavRolloutGenerator:
         self.gpu_id = gpu_id
         self.double_buffered = bool(double_buffered)
         cfg = _lib.Config(num_environments, num_active_scenes, int(self.double_buffered), reset_mode, seed, gpu_id,
-                          max_steps)
+                          max_steps, self.TASK)
         h = C.c_void_p()
         _lib.check(self._L.bpsx_create(C.byref(cfg), C.byref(h)))
         self._h = h
@@ -165,7 +169,7 @@ class PointNavRolloutGenerator:
             t = bps_pytorch.tensor_from_pointer
             self._views[group_idx] = dict(
                 rewards=t(o.rewards, (n,), torch.float32, d, self), masks=t(o.masks, (n,), torch.uint8, d, self),
-                infos=t(o.infos, (n, 3), torch.float32, d, self), polars=t(o.polars, (n, 2), torch.float32, d, self))
+                infos=t(o.infos, (n, o.info_width), torch.float32, d, self), polars=t(o.polars, (n, 2), torch.float32, d, self))
         return self._views[group_idx]
 
     def get_rewards(self, group_idx):
@@ -175,7 +179,7 @@ class PointNavRolloutGenerator:
         return self._outputs(group_idx)["masks"]
 
     def get_infos(self, group_idx):
-        return InfoView(self._outputs(group_idx)["infos"])
+        return InfoView(self._outputs(group_idx)["infos"], self.INFO_FIELDS)
 
     def get_polars(self, group_idx):
         return self._outputs(group_idx)["polars"]
@@ -257,6 +261,20 @@ class PointNavRolloutGenerator:
         xyz, ref = np.zeros((n, 3), np.float32), np.zeros(n, np.uint32)
         _lib.check(self._L.bpsx_random_points(self._h, scene, u.ctypes.data, n, xyz.ctypes.data, ref.ctypes.data))
         return xyz, ref
+
+
+class FleeRolloutGenerator(PointNavRolloutGenerator):
+    """bps_sim.FleeRolloutGenerator (simulator.cpp:830-887, 1818-1819): info = geodesic distance
+    from the episode's start point, reward = its increase per step."""
+    TASK = 1
+    INFO_FIELDS = ("distanceFromStart",)
+
+
+class ExplorationRolloutGenerator(PointNavRolloutGenerator):
+    """bps_sim.ExplorationRolloutGenerator (simulator.cpp:889-997, 1821-1822): info = number of
+    1 m cells (in the start pose's frame) entered so far minus one, reward = 0.25 per new cell."""
+    TASK = 2
+    INFO_FIELDS = ("numVisited",)
 
 
 def nav_only(scenes_blobs, gpu_id=0):

@@ -97,6 +97,12 @@ struct AgentArrays {
   uint32_t* flags;    // [N] transient per-step bits, see kAgent*
   uint32_t* dist_ok;  // [N] 1 when info_prev is the goal->agent distance of the current navmesh point
   float* geo;         // [2N] geodesic results: [i] step query of agent i, [N + i] its reset query
+  // Exploration task only
+  float* exp_init;    // [N][3] position at reset
+  float* exp_inv;     // [N][4] inverse of the rotation at reset
+  int32_t* exp_cells; // [N][cell_cap][3] cells entered this episode
+  uint32_t* exp_count;// [N]
+  uint32_t cell_cap;  // one cell per step at most: max_steps
   // outputs
   float* rewards;     // [N]
   uint8_t* masks;     // [N]

@@ -83,6 +83,7 @@ struct bpsx_sim {
     if (rc == BPSX_OK) owned.push_back((void*)*p);
     return rc;
   }
+  uint32_t info_width() const { return cfg.task == BPSX_TASK_POINTNAV ? 3u : 1u; }
   StepParams params(uint32_t group) const {
     StepParams P{};
     P.n = envs_per_group;
@@ -90,6 +91,8 @@ struct bpsx_sim {
     P.total = cfg.num_environments;
     P.max_steps = (float)(cfg.max_steps ? cfg.max_steps : BPSX_MAX_STEPS);
     P.reset_mode = cfg.reset_mode;
+    P.task = cfg.task;
+    P.info_width = info_width();
     P.seed = cfg.seed;
     memcpy(P.turn_left, turn_left, 16);
     memcpy(P.turn_right, turn_right, 16);
@@ -110,6 +113,9 @@ int bpsx_create(const bpsx_config* cfg, bpsx_sim** out) {
   if (cfg->num_active_scenes % groups != 0)
     return fail(BPSX_E_INVAL, "create: num_active_scenes is not a multiple of the number of groups");
   if (cfg->reset_mode > BPSX_RESET_SAMPLED) return fail(BPSX_E_INVAL, "create: unknown reset_mode");
+  if (cfg->task > BPSX_TASK_EXPLORATION) return fail(BPSX_E_INVAL, "create: unknown task");
+  if (cfg->task == BPSX_TASK_EXPLORATION && cfg->max_steps > 8192)
+    return fail(BPSX_E_UNSUPPORTED, "create: the exploration task keeps one cell per step, max_steps <= 8192");
   int ndev = 0;
   HIP_TRY(hipGetDeviceCount(&ndev));
   if (cfg->gpu_id < 0 || cfg->gpu_id >= ndev) return fail(BPSX_E_INVAL, "create: gpu_id out of range");
@@ -194,9 +200,15 @@ int bpsx_finalize(bpsx_sim* sim) {
       (rc = sim->alloc(&A.cum, N)) || (rc = sim->alloc(&A.init, N)) || (rc = sim->alloc(&A.rew_prev, N)) ||
       (rc = sim->alloc(&A.step, N)) || (rc = sim->alloc(&A.scene, N)) || (rc = sim->alloc(&A.episode, N)) ||
       (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.dist_ok, N)) || (rc = sim->alloc(&A.geo, 2 * N)) ||
-      (rc = sim->alloc(&A.rewards, N)) || (rc = sim->alloc(&A.masks, N)) || (rc = sim->alloc(&A.infos, N * 3)) ||
+      (rc = sim->alloc(&A.rewards, N)) || (rc = sim->alloc(&A.masks, N)) || (rc = sim->alloc(&A.infos, N * sim->info_width())) ||
       (rc = sim->alloc(&A.polars, N * 2)))
     return rc;
+  if (sim->cfg.task == BPSX_TASK_EXPLORATION) {
+    A.cell_cap = sim->cfg.max_steps ? sim->cfg.max_steps : BPSX_MAX_STEPS;
+    if ((rc = sim->alloc(&A.exp_init, N * 3)) || (rc = sim->alloc(&A.exp_inv, N * 4)) ||
+        (rc = sim->alloc(&A.exp_cells, N * (size_t)A.cell_cap * 3)) || (rc = sim->alloc(&A.exp_count, N)))
+      return rc;
+  }
   {
     // env -> scene: contiguous blocks of N / scenes (simulator.cpp:1205-1221, 1578-1592)
     std::vector<uint32_t> scene(N);
@@ -330,7 +342,8 @@ int bpsx_get_outputs(bpsx_sim* sim, uint32_t group, bpsx_outputs* out) {
   const size_t b = (size_t)group * sim->envs_per_group;
   out->rewards = sim->A.rewards + b;
   out->masks = sim->A.masks + b;
-  out->infos = sim->A.infos + b * 3;
+  out->infos = sim->A.infos + b * sim->info_width();
+  out->info_width = sim->info_width();
   out->polars = sim->A.polars + b * 2;
   out->n = sim->envs_per_group;
   return BPSX_OK;

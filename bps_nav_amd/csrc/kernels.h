@@ -21,6 +21,8 @@ struct StepParams {
   uint32_t total;      // agents in the simulator (reset results live at geo[total + i])
   float max_steps;
   uint32_t reset_mode;
+  uint32_t task;       // BPSX_TASK_*
+  uint32_t info_width; // floats per agent in the infos output
   uint64_t seed;
   float turn_left[4], turn_right[4];  // glm::angleAxis(+-radians(10), up), x,y,z,w
   uint32_t* error_flag;

@@ -12,8 +12,13 @@
 //                                                        (PathFinder.cpp:485-541)
 //   step_finish    lane per agent: info, reward, mask from the terminal transition, then the
 //                  new episode's distance bookkeeping    (simulator.cpp:634-641, 758-822, 749-755)
+// The Flee and Exploration tasks (simulator.cpp:830-997) run through the same four launches:
+// Flee keeps the episode's start point where PointNav keeps the snapped goal, so its
+// "distance from start" is the same start-point -> agent query; Exploration makes no queries
+// and keeps its visited cells per agent in HBM.
 #include <hip/hip_runtime.h>
 
+#include "../../include/bpsx.h"
 #include "geodesic_device.h"
 #include "kernels.h"
 
@@ -84,6 +89,26 @@ BPSX_DEV uint32_t wave_append(bool pred, uint32_t* counter) {
 
 BPSX_DEV void load3(const float* p, size_t i, float* o) { o[0] = p[i * 3]; o[1] = p[i * 3 + 1]; o[2] = p[i * 3 + 2]; }
 BPSX_DEV void store3(float* p, size_t i, const float* v) { p[i * 3] = v[0]; p[i * 3 + 1] = v[1]; p[i * 3 + 2] = v[2]; }
+
+// Exploration::InfoFunctor::update (simulator.cpp:897-904): the cell of the agent in the frame
+// of the episode's start pose joins the episode's set.  Returns the set's size.
+BPSX_DEV uint32_t visit_cell(const AgentArrays& A, uint32_t gi, const float* pos) {
+  float ip[3], iq[4];
+  load3(A.exp_init, gi, ip);
+  for (int k = 0; k < 4; ++k) iq[k] = A.exp_inv[(size_t)gi * 4 + k];
+  const float d[3] = {pos[0] - ip[0], pos[1] - ip[1], pos[2] - ip[2]};
+  float g[3];
+  quat_rotate(iq, d, g);
+  const int32_t c0 = (int32_t)(g[0] / 1.0f), c1 = (int32_t)(g[1] / 1.0f), c2 = (int32_t)(g[2] / 1.0f);
+  int32_t* cells = A.exp_cells + (size_t)gi * A.cell_cap * 3;
+  const uint32_t n = A.exp_count[gi];
+  for (uint32_t i = 0; i < n; ++i)
+    if (cells[i * 3] == c0 && cells[i * 3 + 1] == c1 && cells[i * 3 + 2] == c2) return n;
+  if (n >= A.cell_cap) return n;   // cannot happen: one update per step and per reset
+  cells[n * 3] = c0; cells[n * 3 + 1] = c1; cells[n * 3 + 2] = c2;
+  A.exp_count[gi] = n + 1;
+  return n + 1;
+}
 
 __global__ void k_clear_queues(StepQueues Q) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
@@ -173,9 +198,22 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         }
         write_polar(A, gi, pos, rot, goal);
       }
-      const bool reuse = (done || moved) && samePoint && A.dist_ok[gi] != 0;
+      // PointNav measures the distance on every move and at the end of the episode, Flee on
+      // moves only, Exploration never (simulator.cpp:758-790, 845-856, 918-927)
+      const bool measure = P.task == BPSX_TASK_POINTNAV ? (done || moved) : (P.task == BPSX_TASK_FLEE && moved);
+      const bool reuse = measure && samePoint && A.dist_ok[gi] != 0;
       A.flags[gi] = (done ? kAgentDone : 0u) | (moved ? kAgentMoved : 0u) | (reuse ? kAgentReuse : 0u);
-      if ((done || moved) && !reuse) {
+      if (P.task == BPSX_TASK_EXPLORATION) {
+        // the count is taken before the pose arrays move on to the next episode
+        uint32_t cnt = A.exp_count[gi];
+        if (moved) {
+          float pos[3];
+          load3(A.pos, gi, pos);
+          cnt = visit_cell(A, gi, pos);
+        }
+        A.geo[gi] = (float)(cnt - 1);
+      }
+      if (measure && !reuse) {
         want = true;
         load3(A.goal_xyz, gi, q.a);
         q.a_ref = A.goal_ref[gi];
@@ -216,6 +254,34 @@ __global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P
   const uint32_t f = A.flags[gi];
   if (f & kAgentSkip) return;
   const bool done = f & kAgentDone, moved = f & kAgentMoved;
+  if (P.task != BPSX_TASK_POINTNAV) {
+    if (!(f & kAgentResetOnly)) {
+      float v, reward;
+      if (P.task == BPSX_TASK_FLEE) {
+        v = A.info_prev[gi];
+        if (moved) {
+          if (!(f & kAgentReuse)) v = A.geo[gi];
+          A.info_prev[gi] = v;
+          A.dist_ok[gi] = 1;
+        }
+        reward = v - A.rew_prev[gi];
+      } else {
+        v = A.geo[gi];
+        reward = (float)(0.25 * (double)(v - A.rew_prev[gi]));
+      }
+      A.rew_prev[gi] = v;
+      A.rewards[gi] = reward;
+      A.masks[gi] = done ? 0 : 1;
+      A.infos[gi] = v;
+    }
+    if (done || (f & kAgentResetOnly)) {
+      // Flee: distance 0 at the start; Exploration: the start cell is in the set (count 1)
+      A.info_prev[gi] = 0.0f;
+      A.rew_prev[gi] = 0.0f;
+      A.dist_ok[gi] = 0;
+    }
+    return;
+  }
   if (!(f & kAgentResetOnly)) {
     float dist, success = 0, spl = 0;
     const float fresh = (f & kAgentReuse) ? A.info_prev[gi] : A.geo[gi];
@@ -287,6 +353,28 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
     load3(A.goal, gi, goal);
     for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
     const NavPt a = snap_point_wave(nav, s, pos[0], pos[1], pos[2], lds, &cands);
+    if (P.task != BPSX_TASK_POINTNAV) {
+      // no goal snap and no first query (simulator.cpp:838-843, 906-916)
+      if (lane == 0) {
+        const float axyz[3] = {a.x, a.y, a.z}, zero[3] = {0, 0, 0};
+        store3(A.nav_xyz, gi, axyz);
+        A.nav_ref[gi] = a.ref;
+        const bool flee = P.task == BPSX_TASK_FLEE;
+        store3(A.goal_xyz, gi, flee ? axyz : zero);   // Flee: navmeshStart_
+        A.goal_ref[gi] = flee ? a.ref : 0u;
+        write_polar(A, gi, pos, rot, goal);
+        if (!flee) {
+          // glm::inverse(q) = conjugate(q) / dot(q, q)
+          const float d = (rot[3] * rot[3] + rot[0] * rot[0]) + (rot[1] * rot[1] + rot[2] * rot[2]);
+          const float inv[4] = {-rot[0] / d, -rot[1] / d, -rot[2] / d, rot[3] / d};
+          for (int k = 0; k < 4; ++k) A.exp_inv[(size_t)gi * 4 + k] = inv[k];
+          store3(A.exp_init, gi, pos);
+          A.exp_count[gi] = 0;
+          visit_cell(A, gi, pos);
+        }
+      }
+      continue;
+    }
     const NavPt b = snap_point_wave(nav, s, goal[0], goal[1], goal[2], lds, &cands);
     if (lane == 0) {
       const float axyz[3] = {a.x, a.y, a.z}, bxyz[3] = {b.x, b.y, b.z};

@@ -47,6 +47,18 @@ extern "C" {
 #define BPSX_RESET_EPISODES 0
 #define BPSX_RESET_SAMPLED 1
 
+/* Tasks = the reference's Simulator instantiations (simulator.cpp:1811-1823): what info and
+ * reward are computed per step.  The agent dynamics, episodes and polar observation are the
+ * same for all three.
+ *   POINTNAV     info {success, spl, distanceToGoal}, reward per simulator.cpp:737-825
+ *   FLEE         info {distanceFromStart} = geodesic(start point -> agent), refreshed on forward
+ *                moves; reward = its increase (simulator.cpp:830-887)
+ *   EXPLORATION  info {numVisited} = 1 m cells of the start pose's frame entered so far, minus
+ *                one; reward = 0.25 per new cell (simulator.cpp:889-997) */
+#define BPSX_TASK_POINTNAV 0
+#define BPSX_TASK_FLEE 1
+#define BPSX_TASK_EXPLORATION 2
+
 typedef struct bpsx_sim bpsx_sim;
 
 /* Mirrors the constructor arguments of bps_sim.PointNavRolloutGenerator that reach
@@ -59,6 +71,7 @@ typedef struct bpsx_config {
   uint64_t seed;              /* seeds the per-(env, reset#) counter-based stream          */
   int32_t gpu_id;             /* HIP device ordinal                                        */
   uint32_t max_steps;         /* 0 => BPSX_MAX_STEPS                                       */
+  uint32_t task;              /* BPSX_TASK_*                                               */
 } bpsx_config;
 
 /* Output tensors of one group, device pointers that stay valid and fixed for the
@@ -66,9 +79,11 @@ typedef struct bpsx_config {
 typedef struct bpsx_outputs {
   float *rewards;  /* f32[n]                                   */
   uint8_t *masks;  /* u8[n], 1 = episode continues, 0 = done   */
-  float *infos;    /* f32[n][3] = success, spl, distanceToGoal */
+  float *infos;    /* f32[n][info_width]: PointNav success, spl, distanceToGoal;
+                      Flee distanceFromStart; Exploration numVisited */
   float *polars;   /* f32[n][2] = rho, -phi                    */
   uint32_t n;      /* envs in this group                       */
+  uint32_t info_width; /* floats per env in infos: 3 for PointNav, 1 otherwise */
 } bpsx_outputs;
 
 /* Per-agent state of one group, device pointers, for parity harnesses. */

@@ -128,6 +128,7 @@ struct ApiImpl {
   BPO_API int bpo_sim_add_scene(void* h, const void* b, size_t n, const float* ep, uint32_t E) {           \
     return ApiImpl<B>::sim_add_scene(h, b, n, ep, E);                                                       \
   }                                                                                                         \
+  BPO_API void bpo_sim_set_task(void* h, uint32_t task) { ((ApiImpl<B>::SimT*)h)->setTask(task); }         \
   BPO_API int bpo_sim_finalize(void* h) { return ApiImpl<B>::sim_finalize(h); }                             \
   BPO_API uint32_t bpo_sim_envs_per_group(void* h) { return ((ApiImpl<B>::SimT*)h)->envsPerGroup(); }      \
   BPO_API void bpo_sim_reset(void* h, uint32_t g) { ((ApiImpl<B>::SimT*)h)->reset(g); }                    \

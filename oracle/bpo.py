@@ -45,6 +45,7 @@ class Lib:
         L.bpo_sim_create.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int]
         L.bpo_sim_add_scene.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t, _f32p, C.c_uint32]
         L.bpo_sim_finalize.argtypes = [C.c_void_p]
+        L.bpo_sim_set_task.argtypes = [C.c_void_p, C.c_uint32]
         L.bpo_sim_envs_per_group.argtypes = [C.c_void_p]
         L.bpo_sim_envs_per_group.restype = C.c_uint32
         L.bpo_sim_reset.argtypes = [C.c_void_p, C.c_uint32]
@@ -150,9 +151,12 @@ class Nav:
 class Sim:
     """CPU simulator with the reference's worker-thread dispatch."""
 
-    def __init__(self, lib, scenes, num_envs, double_buffered=False, reset_mode=0, seed=0, max_steps=0, threads=1):
+    def __init__(self, lib, scenes, num_envs, double_buffered=False, reset_mode=0, seed=0, max_steps=0, threads=1,
+                 task=0):
+        """task: 0 PointNav, 1 Flee, 2 Exploration (infos column 0 holds the single info value of 1 and 2)."""
         self.lib = lib
         self.h = lib.L.bpo_sim_create(num_envs, len(scenes), int(double_buffered), reset_mode, seed, max_steps, threads)
+        lib.L.bpo_sim_set_task(self.h, task)
         for blob, eps in scenes:
             eps = np.ascontiguousarray(eps, np.float32).reshape(-1, 10)
             if lib.L.bpo_sim_add_scene(self.h, blob, len(blob), eps, len(eps)) != 0:

@@ -5,17 +5,22 @@
 // absent), so this file follows it by reading:
 //   BaseSimulator::reset/step/handleMovement/updateObservationState  simulator.cpp:601-710
 //   PointNav::InfoFunctor / RewardFunctor                            simulator.cpp:737-825
+//   Flee::InfoFunctor / RewardFunctor                                simulator.cpp:830-887
+//   Exploration::InfoFunctor / RewardFunctor                         simulator.cpp:889-997
 //   computeGeoDist                                                   simulator.cpp:553-563
 //   RolloutGenerator::simulate / simulateStart / simulateEnd         simulator.cpp:1619-1700
 //   EnvironmentGroup env->scene assignment                           simulator.cpp:1205-1221
 // glm closed forms (angleAxis, quat*quat, quat*vec3, mat3_cast) are written out; glm is
 // not vendored by the reference, so those are "parity unpinned" and pinned here by closed
-// forms in tests/test_oracle_closed_forms.py.
+// forms in tests/test_oracle_closed_forms.py.  The same holds for glm::inverse(quat) =
+// conjugate / dot with dot = (w*w + x*x) + (y*y + z*z) (glm 0.9.9 compute_dot for quaternions),
+// used by the Exploration task: parity unpinned, pinned by closed forms.
 //
 // Deviation by design: the reference draws the reset episode from a per-thread mt19937
 // claimed racily by worker threads (simulator.cpp:605-607, 1626, 1736); this build defines a
 // counter-based stream keyed by (seed, env index, reset count) so resets are reproducible.
 #pragma once
+#include <array>
 #include <atomic>
 #include <cmath>
 #include <condition_variable>
@@ -32,6 +37,7 @@ constexpr float SUCCESS_REWARD = 2.5f;
 constexpr float SLACK_REWARD = 1e-2f;
 constexpr float SUCCESS_DISTANCE = 0.2f;
 constexpr float FORWARD_STEP_SIZE = 0.25f;
+enum Task : uint32_t { TASK_POINTNAV = 0, TASK_FLEE = 1, TASK_EXPLORATION = 2 };
 
 struct NavPt {
   float xyz[3];
@@ -104,7 +110,15 @@ struct Env {
   float infoPrevDist = 0, cumDist = 0, initDist = 0, prevPos[3] = {0, 0, 0};
   float rewardPrevDist = 0;
   uint32_t episode = 0, numResets = 0;
+  // Exploration: cells visited, in the frame of the episode's start pose
+  float initPos[3] = {0, 0, 0}, invInitRot[4] = {0, 0, 0, 1};
+  std::vector<std::array<int, 3>> visited;
 };
+// glm::inverse(quat): conjugate(q) / dot(q, q)
+inline void quat_inverse(const float* q, float* o) {
+  const float d = (q[3] * q[3] + q[0] * q[0]) + (q[1] * q[1] + q[2] * q[2]);
+  o[3] = q[3] / d; o[0] = -q[0] / d; o[1] = -q[1] / d; o[2] = -q[2] / d;
+}
 
 struct SceneEpisodes {
   std::vector<float> rows;  // [E][10]
@@ -127,6 +141,7 @@ class Sim {
       : numEnvs_(numEnvs), numScenes_(numScenes), groups_(doubleBuffered ? 2 : 1), resetMode_(resetMode),
         seed_(seed), maxSteps_(maxSteps ? maxSteps : 500), numThreads_(numThreads < 1 ? 1 : numThreads) {}
   ~Sim() { stopWorkers(); }
+  void setTask(uint32_t task) { task_ = task; }
 
   bool addScene(const uint8_t* bytes, size_t n, const float* episodes, uint32_t numEpisodes, std::string* err) {
     auto s = B::load(bytes, n, err);
@@ -216,6 +231,23 @@ class Sim {
     memcpy(e.goal, ep + 7, 12);
     e.nav = c.snap(e.scene, e.pos);
     updateObservation(gi);
+    if (task_ == TASK_FLEE) {
+      // Flee::InfoFunctor::reset: the start point is kept where PointNav keeps the goal point
+      e.navGoal = e.nav;
+      e.infoPrevDist = 0.0f;
+      e.rewardPrevDist = 0.0f;
+      return;
+    }
+    if (task_ == TASK_EXPLORATION) {
+      e.navGoal = NavPt{{0, 0, 0}, 0};
+      e.visited.clear();
+      memcpy(e.initPos, e.pos, 12);
+      quat_inverse(e.rot, e.invInitRot);
+      visit(e);
+      e.infoPrevDist = (float)(e.visited.size() - 1);
+      e.rewardPrevDist = e.infoPrevDist;
+      return;
+    }
     // InfoFunctor::reset
     e.navGoal = c.snap(e.scene, e.goal);
     e.cumDist = 0;
@@ -224,6 +256,16 @@ class Sim {
     memcpy(e.prevPos, e.pos, 12);
     // RewardFunctor::reset
     e.rewardPrevDist = e.infoPrevDist;
+  }
+  // Exploration::InfoFunctor::update
+  static void visit(Env& e) {
+    const float d[3] = {e.pos[0] - e.initPos[0], e.pos[1] - e.initPos[1], e.pos[2] - e.initPos[2]};
+    float g[3];
+    quat_rotate(e.invInitRot, d, g);
+    const std::array<int, 3> cell = {(int)(g[0] / 1.0f), (int)(g[1] / 1.0f), (int)(g[2] / 1.0f)};
+    for (const auto& v : e.visited)
+      if (v == cell) return;
+    e.visited.push_back(cell);
   }
   bool stepEnv(uint32_t gi, int64_t action, typename B::Ctx& c) {
     Env& e = envs_[gi];
@@ -252,6 +294,24 @@ class Sim {
         quat_mul(e.rot, turns_.right, e.rot);
       }
       updateObservation(gi);
+    }
+    if (task_ != TASK_POINTNAV) {
+      float v;
+      if (task_ == TASK_FLEE) {
+        if (e.updated) e.infoPrevDist = c.geodesic(e.scene, e.navGoal, e.nav);
+        v = e.infoPrevDist;
+        rewards_[gi] = v - e.rewardPrevDist;
+      } else {
+        if (e.updated) visit(e);
+        v = (float)(e.visited.size() - 1);
+        rewards_[gi] = (float)(0.25 * (double)(v - e.rewardPrevDist));
+      }
+      e.rewardPrevDist = v;
+      masks_[gi] = done ? 0 : 1;
+      infos_[(size_t)gi * 3 + 0] = v;
+      infos_[(size_t)gi * 3 + 1] = 0;
+      infos_[(size_t)gi * 3 + 2] = 0;
+      return done;
     }
     // InfoFunctor::step
     float dist = 0, success = 0, spl = 0;
@@ -339,6 +399,7 @@ class Sim {
     workers_.clear();
   }
 
+  uint32_t task_ = TASK_POINTNAV;
   uint32_t numEnvs_, numScenes_, groups_, resetMode_;
   uint64_t seed_;
   uint32_t maxSteps_;

@@ -144,6 +144,47 @@ def test_step_parity(oracle, torch_cuda, config, num_scenes, n, steps, mode):
     gen.close()
 
 
+@pytest.mark.parametrize("task,config,num_scenes,n,steps,mode,max_steps", [
+    (1, 2, 4, 256, 250, 0, 60), (1, 4, 2, 128, 120, 1, 0), (2, 3, 2, 128, 250, 0, 80), (2, 1, 1, 64, 150, 1, 0)])
+def test_flee_and_exploration_step_parity(oracle, torch_cuda, task, config, num_scenes, n, steps, mode, max_steps):
+    """The other two tasks of the reference (simulator.cpp:830-997) against the oracle: same
+    dynamics, info = distance from start (Flee) or visited-cell count (Exploration)."""
+    from bps_nav_amd import bps_sim
+    from oracle import bpo
+    print(f"case: task {task} config {config} scenes {num_scenes} agents {n} mode {mode}", flush=True)
+    sc = common.build_scenes(oracle, config, num_scenes)
+    cpu = bpo.Sim(oracle, sc, n, reset_mode=mode, seed=23, threads=4, task=task, max_steps=max_steps)
+    cls = bps_sim.FleeRolloutGenerator if task == 1 else bps_sim.ExplorationRolloutGenerator
+    gen = cls("", "", n, len(sc), scenes=sc, reset_mode=mode, seed=23, max_steps=max_steps)
+    cpu.reset()
+    gen.reset(0)
+    infos = gen.get_infos(0)
+    assert infos.dtype.names == (("distanceFromStart",) if task == 1 else ("numVisited",))
+    assert infos.packed.shape == (n, 1)
+    rewards, masks, state = gen.get_rewards(0), gen.get_masks(0), gen.get_state(0)
+    dones = 0
+    nonzero = 0
+    for t, a in enumerate(common.action_stream(config, steps, n)):
+        cpu.step(a)
+        gen.step(0, a)
+        co, cs = cpu.outputs(), cpu.state()
+        g_state = {k: v.cpu().numpy() for k, v in state.items()}
+        for k in ("poly_ref", "goal_ref", "step", "episode", "num_resets"):
+            assert np.array_equal(cs[k], g_state[k].view(np.uint32)), f"{k} differs at step {t}"
+        assert np.array_equal(common.bits(g_state["position"]), common.bits(cs["position"])), f"position bits at step {t}"
+        assert np.array_equal(co["masks"], masks.cpu().numpy()), f"dones differ at step {t}"
+        gi = infos.packed.cpu().numpy()[:, 0]
+        gr = rewards.cpu().numpy()
+        np.testing.assert_allclose(gi, co["infos"][:, 0], rtol=1e-3, atol=0, equal_nan=True)
+        np.testing.assert_allclose(gr, co["rewards"], rtol=1e-3, atol=1e-6, equal_nan=True)
+        assert np.array_equal(common.bits(gi), common.bits(co["infos"][:, 0])), f"info bits at step {t}"
+        dones += int((co["masks"] == 0).sum())
+        nonzero += int((gr != 0).sum())
+    assert dones > 0 and nonzero > 0
+    gen.check_errors()
+    gen.close()
+
+
 def test_error_paths(oracle, torch_cuda):
     print("case: error paths", flush=True)
     sc = common.build_scenes(oracle, 1, 1, episodes_per_scene=8)

@@ -189,10 +189,10 @@ def test_sampling_matches_reference_distribution(oracle, reflib):
 
 
 # ---------------------------------------------------------------- state machine algebra
-def one_room_sim(oracle, n=1, max_steps=0, start=(2, 0, 2), goal=(2, 0, 8), yaw=0.0):
+def one_room_sim(oracle, n=1, max_steps=0, start=(2, 0, 2), goal=(2, 0, 8), yaw=0.0, task=0):
     blob = meshes.l_shape()
     ep = np.concatenate([start, episodes.yaw_quat(np.array(yaw)), goal]).astype(np.float32)[None]
-    return bpo.Sim(oracle, [(blob, ep)], n, max_steps=max_steps)
+    return bpo.Sim(oracle, [(blob, ep)], n, max_steps=max_steps, task=task)
 
 
 def test_forward_moves_along_heading_and_rewards_progress(oracle):
@@ -274,6 +274,71 @@ def test_episode_ends_at_max_steps_and_reward_sum_telescopes(oracle):
     # step pays no progress term
     assert last_d == pytest.approx(init - 0.25 * 11, abs=1e-4)
     assert total == pytest.approx((init - (init - 0.25 * 10)) - 0.01 * 11, abs=1e-4)
+
+
+def test_flee_distance_from_start_and_reward(oracle):
+    # Flee (simulator.cpp:830-887): info = geodesic(start point -> agent), refreshed on forward
+    # moves only; reward = its change, no slack, no success bonus
+    sim = one_room_sim(oracle, yaw=math.pi, task=1, max_steps=9)
+    sim.reset()
+    assert sim.outputs()["infos"][0, 0] == 0.0
+    for k in range(1, 5):
+        sim.step(np.array([1]))
+        o = sim.outputs()
+        assert o["infos"][0, 0] == pytest.approx(0.25 * k, abs=1e-5)   # one convex room: straight line
+        assert o["rewards"][0] == pytest.approx(0.25, abs=1e-5) and o["masks"][0] == 1
+    sim.step(np.array([2]))      # a turn: distance kept, reward 0
+    o = sim.outputs()
+    assert o["infos"][0, 0] == pytest.approx(1.0, abs=1e-5) and o["rewards"][0] == 0.0
+    sim.step(np.array([3])); sim.step(np.array([3]))
+    sim.step(np.array([0]))      # stop: done, distance kept (not recomputed), reward 0, then reset
+    o = sim.outputs()
+    assert o["masks"][0] == 0 and o["infos"][0, 0] == pytest.approx(1.0, abs=1e-5) and o["rewards"][0] == 0.0
+    assert sim.state()["num_resets"][0] == 2 and sim.state()["step"][0] == 1
+    sim.step(np.array([1]))      # new episode measures from the new start: prev = 0
+    assert sim.outputs()["rewards"][0] == pytest.approx(0.25, abs=1e-5)
+
+
+def test_exploration_counts_cells_of_the_start_frame(oracle):
+    # Exploration (simulator.cpp:889-997): 1 m cells of the start pose's frame, int() truncation,
+    # so walking straight ahead along -z' enters a new cell when the path length reaches 1, 2, ...
+    for yaw in (math.pi, math.pi - 0.3):
+        sim = one_room_sim(oracle, yaw=yaw, task=2, start=(2, 0, 2.5))
+        sim.reset()
+        assert sim.outputs()["infos"][0, 0] == 0.0
+        seen = []
+        for k in range(1, 15):
+            sim.step(np.array([1]))
+            o = sim.outputs()
+            seen.append(o["infos"][0, 0])
+            if k % 4 != 0:     # away from the exact cell boundaries
+                assert o["infos"][0, 0] == float(k // 4), (yaw, k, seen)
+        assert seen[-1] == 3.0
+        # rewards: 0.25 per new cell, summed = 0.25 * cells
+        # turning on the spot or revisiting adds nothing
+        for a in (2, 2, 3, 3):
+            sim.step(np.array([a]))
+            assert sim.outputs()["rewards"][0] == 0.0 and sim.outputs()["infos"][0, 0] == 3.0
+    # 18 left turns then forward: back over visited cells, count unchanged
+    for _ in range(18):
+        sim.step(np.array([2]))
+    for _ in range(6):
+        sim.step(np.array([1]))
+        assert sim.outputs()["infos"][0, 0] == 3.0
+    sim.step(np.array([0]))
+    assert sim.outputs()["masks"][0] == 0 and sim.outputs()["infos"][0, 0] == 3.0
+    sim.step(np.array([1]))
+    assert sim.outputs()["infos"][0, 0] == 0.0 and sim.outputs()["rewards"][0] == 0.0
+
+
+def test_exploration_reward_is_quarter_per_new_cell(oracle):
+    sim = one_room_sim(oracle, yaw=math.pi, task=2, start=(2, 0, 2.4))
+    sim.reset()
+    total = 0.0
+    for _ in range(13):
+        sim.step(np.array([1]))
+        total += sim.outputs()["rewards"][0]
+    assert total == pytest.approx(0.25 * sim.outputs()["infos"][0, 0]) and sim.outputs()["infos"][0, 0] == 3.0
 
 
 def test_invalid_action_is_flagged_and_agent_untouched(oracle):
