@@ -96,6 +96,7 @@ struct AgentArrays {
   uint32_t* nresets;  // [N]
   uint32_t* flags;    // [N] transient per-step bits, see kAgent*
   uint32_t* dist_ok;  // [N] 1 when info_prev is the goal->agent distance of the current navmesh point
+  uint32_t* last_cost;// [N] nodes expanded by the agent's most recent path search (scheduling hint)
   float* geo;         // [2N] geodesic results: [i] step query of agent i, [N + i] its reset query
   // Exploration task only
   float* exp_init;    // [N][3] position at reset
@@ -151,7 +152,19 @@ struct GeoQuery {
   uint32_t b_ref;
   uint32_t scene;
   uint32_t out;   // index into the result array
+  uint32_t cost_slot;  // agent whose cost estimate this query refreshes, or kNoCostSlot
+  uint32_t pad;
 };
+constexpr uint32_t kNoCostSlot = 0xffffffffu;
+
+// Path searches differ in length by two orders of magnitude and each is sequential, so a step
+// ends when its longest search ends.  Queries are therefore queued in classes of expected
+// cost (the nodes the agent's previous search expanded) and the longest class is served
+// first; a search that runs long also raises its wavefront's issue priority.
+constexpr int kGeoClasses = 4;
+inline __host__ __device__ uint32_t geo_class(uint32_t last_cost) {
+  return last_cost >= 1024u ? 0u : last_cost >= 512u ? 1u : last_cost >= 192u ? 2u : 3u;
+}
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,

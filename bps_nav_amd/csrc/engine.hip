@@ -199,7 +199,7 @@ int bpsx_finalize(bpsx_sim* sim) {
       (rc = sim->alloc(&A.goal_ref, N)) || (rc = sim->alloc(&A.prev_pos, N * 3)) || (rc = sim->alloc(&A.info_prev, N)) ||
       (rc = sim->alloc(&A.cum, N)) || (rc = sim->alloc(&A.init, N)) || (rc = sim->alloc(&A.rew_prev, N)) ||
       (rc = sim->alloc(&A.step, N)) || (rc = sim->alloc(&A.scene, N)) || (rc = sim->alloc(&A.episode, N)) ||
-      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.dist_ok, N)) || (rc = sim->alloc(&A.geo, 2 * N)) ||
+      (rc = sim->alloc(&A.nresets, N)) || (rc = sim->alloc(&A.flags, N)) || (rc = sim->alloc(&A.dist_ok, N)) || (rc = sim->alloc(&A.last_cost, N)) || (rc = sim->alloc(&A.geo, 2 * N)) ||
       (rc = sim->alloc(&A.rewards, N)) || (rc = sim->alloc(&A.masks, N)) || (rc = sim->alloc(&A.infos, N * sim->info_width())) ||
       (rc = sim->alloc(&A.polars, N * 2)))
     return rc;
@@ -220,7 +220,7 @@ int bpsx_finalize(bpsx_sim* sim) {
     HIP_TRY(hipMemcpy(A.rot, rot.data(), N * 16, hipMemcpyHostToDevice));
   }
   if ((rc = sim->alloc(&sim->d_error, 1)) || (rc = sim->alloc(&sim->d_counters, BPSX_NUM_COUNTERS))) return rc;
-  if ((rc = sim->alloc(&sim->d_batch_counts, 2))) return rc;
+  if ((rc = sim->alloc(&sim->d_batch_counts, kGeoClasses + 1))) return rc;
 
   // ---- A* wavefronts: as many as the LDS of the device holds at once, not one per agent
   hipDeviceProp_t prop;
@@ -237,9 +237,10 @@ int bpsx_finalize(bpsx_sim* sim) {
   sim->groups.resize(sim->num_groups);
   const size_t n = sim->envs_per_group;
   for (auto& g : sim->groups) {
-    if ((rc = sim->alloc(&g.Q.counts, 8)) || (rc = sim->alloc(&g.Q.queries, 2 * n)) ||
+    if ((rc = sim->alloc(&g.Q.counts, 8)) || (rc = sim->alloc(&g.Q.queries, (size_t)kGeoClasses * 2 * n)) ||
         (rc = sim->alloc(&g.Q.reset_list, n)) || (rc = sim->alloc(&g.d_actions, n)))
       return rc;
+    g.Q.stride = (uint32_t)(2 * n);
     HIP_TRY(hipHostMalloc((void**)&g.h_actions, n * sizeof(int64_t), hipHostMallocDefault));
     HIP_TRY(hipEventCreateWithFlags(&g.done, hipEventDisableTiming));
     for (auto& e : g.ev) HIP_TRY(hipEventCreate(&e));

@@ -61,6 +61,13 @@ BPSX_DEV void wave_sync() {
 // Keeps the compiler from folding an LDS access and an HBM access of two branches into one
 // generic-address access (which would wait on both memory counters and on pending stores).
 #define BPSX_KEEP_APART() asm volatile("")
+// s_setprio takes an immediate
+BPSX_DEV void set_wave_priority(int p) {
+  if (p >= 3) __builtin_amdgcn_s_setprio(3);
+  else if (p == 2) __builtin_amdgcn_s_setprio(2);
+  else if (p == 1) __builtin_amdgcn_s_setprio(1);
+  else __builtin_amdgcn_s_setprio(0);
+}
 BPSX_DEV int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
 BPSX_DEV float uniform_f(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 BPSX_DEV float lane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
@@ -113,6 +120,7 @@ struct GeoWave {
   int heapSize;
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
+  int basePrio;                      // issue priority the query started with
 
   // ---------------------------------------------------------------- node pool
   template <bool S> BPSX_DEV uint32_t link(int i) const {
@@ -257,11 +265,32 @@ struct RegHeap {
     }
     set(q, t, n);
   }
+  // Below 64 entries (almost always) only the first register pair is in use and the walks
+  // need no pair selection.
+  BPSX_DEV void bubble_up_small(int q, uint32_t t, uint32_t n) {
+    while (q > 1) {
+      const int p = q >> 1;
+      const uint32_t pt = rlane(t0, p);
+      if (!(pt > t)) break;
+      const uint32_t pn = rlane(n0, p);
+      t0 = wlane(t0, pt, q);
+      n0 = wlane(n0, pn, q);
+      q = p;
+    }
+    t0 = wlane(t0, t, q);
+    n0 = wlane(n0, n, q);
+  }
   BPSX_DEV void push(uint32_t t, uint32_t n) {
     size++;
-    bubble_up(size, t, n);
+    if (size < 64) bubble_up_small(size, t, n);
+    else bubble_up(size, t, n);
   }
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
+    if (size < 64) {
+      const unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);
+      if (m) bubble_up_small(__ffsll((long long)m) - 1, t, n);
+      return;
+    }
     int q = 0;
     unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);
     if (m) q = __ffsll((long long)m) - 1;
@@ -277,7 +306,43 @@ struct RegHeap {
   // Positions past the end hold kEmpty, greater than any total, so the walk needs no bounds.
   static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
   BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
-  BPSX_DEV void pop() {
+  // The same for fewer than 64 entries, done by all lanes at once.  Which child the hole moves
+  // to depends only on the children's keys, which the moves above them do not change: every
+  // lane q picks the smaller child of position q (two cross-lane reads), the hole's route is
+  // read off that table with five dependent lane reads, and then every route position whose
+  // smaller child is not greater than the entry takes that child, and the first one whose
+  // child is greater takes the entry.
+  BPSX_DEV void pop_small(int lane) {
+    const int last = size;
+    size--;
+    const uint32_t lt = rlane(t0, last), ln = rlane(n0, last);
+    t0 = wlane(t0, kEmpty, last);
+    if (size == 0) return;
+    const bool inner = lane < 32;   // positions 32..63 have their children past the pair: none
+    // all lanes take part in the cross-lane reads (an inactive source lane would read as 0)
+    const uint32_t gl = (uint32_t)__builtin_amdgcn_ds_bpermute(lane * 8, (int)t0);
+    const uint32_t gr = (uint32_t)__builtin_amdgcn_ds_bpermute(lane * 8 + 4, (int)t0);
+    const uint32_t cl = inner ? gl : kEmpty, cr = inner ? gr : kEmpty;
+    const bool right = cr < cl;
+    const uint32_t cmin = right ? cr : cl;
+    const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);
+    const uint32_t cn = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(choice * 4), (int)n0);
+    // route of the hole: 1, choice[1], choice[choice[1]], ... while inside the pair
+    unsigned long long route = 2ull;
+    uint32_t q = 1;
+#pragma unroll
+    for (int lvl = 0; lvl < 5; ++lvl) {
+      q = rlane(choice, (int)(q & 31));          // levels 0..4 start from positions below 32
+      route |= 1ull << (q & 63);
+    }
+    const bool on = (route >> lane) & 1ull;
+    const bool take = on && cmin <= lt;
+    const bool land = on && !take && (lane == 1 || t0 <= lt);
+    t0 = take ? cmin : (land ? lt : t0);
+    n0 = take ? cn : (land ? ln : n0);
+  }
+  BPSX_DEV void pop(int lane) {
+    if (size < 64) { pop_small(lane); return; }
     const int last = size;
     size--;
     uint32_t lt, ln;
@@ -308,6 +373,7 @@ struct AstarState {
   int lastBest;
   float lastBestCost;
   bool outOfNodes;
+  int expanded;
   RegHeap rh;
 };
 enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
@@ -353,11 +419,15 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     PHASE_MARK(0);
     if (SH) g.pop<true>();
-    else rh.pop();
+    else rh.pop(lane);
     PHASE_MARK(1);
     g.set_state<S>(bi, 2u | (pidx << 2));   // open -> closed
     if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
     (*pops)++;
+    // a search that runs long gets ahead of the short ones sharing its SIMD
+    if ((++st.expanded & 255) == 0) {
+      set_wave_priority(g.basePrio + (st.expanded >> 8));
+    }
     PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
     int ni = -1;
@@ -381,6 +451,15 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       // hash insertion by all new nodes at once; of two that share a bucket one store wins
       // and the other lane goes round again behind it
       bool pending = isNew && nb != kNoNb;
+      if ((need & (need - 1)) == 0) {   // one new node: no other lane can take its bucket
+        if (pending) {
+          const uint32_t head = L->first[bucket];
+          g.set_link<S>(ni, nb | (head << 16));
+          L->first[bucket] = (uint16_t)ni;
+        }
+        pending = false;
+        wave_sync();
+      }
       while (__ballot(pending)) {
         if (pending) {
           const uint32_t head = L->first[bucket];
@@ -483,8 +562,14 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     wave_sync();
     return 1;
   }
-  g.clear();
   AstarState st;
+  const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kNvp;
+#ifdef BPSX_PHASE_TIMING
+#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0)
+#else
+#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
+#endif
+  g.clear();
   {
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
     const float total = sqrtf(dx * dx + dy * dy + dz * dz) * 0.999f;
@@ -500,18 +585,13 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       L->first[GeoWave::hash(startIp)] = 0;
     }
     wave_sync();
-    st.rh.init();
-    st.rh.push(__float_as_uint(total), 0u);
     st.lastBest = 0;
     st.lastBestCost = total;
     st.outOfNodes = false;
+    st.expanded = 0;
+    st.rh.init();
+    st.rh.push(__float_as_uint(total), 0u);
   }
-  const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kNvp;
-#ifdef BPSX_PHASE_TIMING
-#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0)
-#else
-#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
-#endif
   AstarExit ex = ASTAR_RUN(0);
   if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
   if (ex == kAstarGrowHeap) {

@@ -112,7 +112,8 @@ BPSX_DEV uint32_t visit_cell(const AgentArrays& A, uint32_t gi, const float* pos
 
 __global__ void k_clear_queues(StepQueues Q) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
-    Q.counts[kQGeo] = 0; Q.counts[kQGeoHead] = 0; Q.counts[kQReset] = 0;
+    for (int c = 0; c < kGeoClasses; ++c) Q.counts[kQGeo + c] = 0;
+    Q.counts[kQGeoHead] = 0; Q.counts[kQReset] = 0;
   }
 }
 
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
                                                    const int64_t* __restrict__ actions) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   bool want = false, reset = false;
+  uint32_t cls = 0;
   GeoQuery q{};
   uint32_t movePolys = 0, gi = 0;
   if (i < P.n) {
@@ -221,6 +223,9 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         q.b_ref = A.nav_ref[gi];
         q.scene = A.scene[gi];
         q.out = gi;
+        q.cost_slot = done ? kNoCostSlot : gi;   // a finished episode's search predicts nothing
+        q.pad = 0;
+        cls = geo_class(A.last_cost[gi]);
       }
       if (done) {
         // the terminal query above holds copies of the old episode's points: the pose arrays can
@@ -230,8 +235,11 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
       }
     }
   }
-  const uint32_t slot = wave_append(want, &Q.counts[kQGeo]);
-  if (want) Q.queries[slot] = q;
+  for (uint32_t c = 0; c < (uint32_t)kGeoClasses; ++c) {
+    const bool mine = want && cls == c;
+    const uint32_t slot = wave_append(mine, &Q.counts[kQGeo + c]);
+    if (mine) Q.queries[(size_t)c * Q.stride + slot] = q;
+  }
   const uint32_t rslot = wave_append(reset, &Q.counts[kQReset]);
   if (reset) Q.reset_list[rslot] = gi;
   // counters, one atomic per wavefront
@@ -388,16 +396,24 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
       q.b[0] = b.x; q.b[1] = b.y; q.b[2] = b.z; q.b_ref = b.ref;
       q.scene = A.scene[gi];
       q.out = P.total + gi;
-      Q.queries[atomicAdd(&Q.counts[kQGeo], 1u)] = q;
+      q.cost_slot = gi;
+      q.pad = 0;
+      // a new episode: no history, assume a search of upper-middle length
+      Q.queries[(size_t)1 * Q.stride + atomicAdd(&Q.counts[kQGeo + 1], 1u)] = q;
     }
   }
   if (lane == 0 && blockIdx.x == 0 && n) atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
   if (lane == 0 && cands) atomicAdd((unsigned long long*)&P.counters[kCntSnapCands], (unsigned long long)cands);
 }
 
-__global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries,
-                                                 const uint32_t* __restrict__ count, uint32_t* head, float* out,
-                                                 GeoSlot* slots, uint64_t* counters) {
+#ifdef BPSX_QUERY_TRACE
+// diagnostic build: start/end time (100 MHz wall clock), nodes expanded and class of every query
+__device__ unsigned long long g_trace[1 << 17][4];
+__device__ unsigned int g_trace_n;
+#endif
+__global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
+                                                 const uint32_t* __restrict__ counts, uint32_t* head, float* out,
+                                                 uint32_t* last_cost, GeoSlot* slots, uint64_t* counters) {
   __shared__ GeoShared lds;
   GeoWave g;
   g.lane = (int)threadIdx.x;
@@ -406,7 +422,11 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
   g.heapSize = 0;
   g.nodeCount = 0;
   g.linkSpills = g.heapSpills = 0;
-  const uint32_t nq = *count;
+  // classes are served in order: class c owns ticket numbers [first[c], first[c + 1])
+  uint32_t first[kGeoClasses + 1];
+  first[0] = 0;
+  for (int c = 0; c < kGeoClasses; ++c) first[c + 1] = first[c] + (uint32_t)uniform_i((int)counts[c]);
+  const uint32_t nq = first[kGeoClasses];
   uint32_t pops = 0, corridor = 0, done = 0;
 #ifdef BPSX_PHASE_TIMING
   unsigned long long phase_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -416,13 +436,31 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
     if (g.lane == 0) qi = atomicAdd(head, 1u);
     qi = (uint32_t)uniform_i((int)qi);
     if (qi >= nq) break;
-    const GeoQuery q = queries[qi];
+    int cls = 0;
+    while (qi >= first[cls + 1]) cls++;
+    const GeoQuery q = queries[(size_t)cls * stride + (qi - first[cls])];
+    const uint32_t pops0 = pops;
+#ifdef BPSX_QUERY_TRACE
+    const unsigned long long trace_t0 = wall_clock64();
+#endif
+    g.basePrio = kGeoClasses - 1 - cls;
+    set_wave_priority(g.basePrio);
 #ifdef BPSX_PHASE_TIMING
     const float d = geodesic_query(g, nav, q, &pops, &corridor, phase_acc);
 #else
     const float d = geodesic_query(g, nav, q, &pops, &corridor);
 #endif
-    if (g.lane == 0) out[q.out] = d;
+    if (g.lane == 0) {
+#ifdef BPSX_QUERY_TRACE
+      const unsigned int ti = atomicAdd(&g_trace_n, 1u);
+      if (ti < (1u << 17)) {
+        g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = pops - pops0;
+        g_trace[ti][3] = (unsigned long long)cls | ((unsigned long long)blockIdx.x << 8) | ((unsigned long long)qi << 32);
+      }
+#endif
+      out[q.out] = d;
+      if (last_cost && q.cost_slot != kNoCostSlot) last_cost[q.cost_slot] = pops - pops0;
+    }
     done++;
     wave_sync();
   }
@@ -468,6 +506,7 @@ __global__ void k_make_queries(uint32_t scene, const float* sxyz, const uint32_t
   GeoQuery o;
   for (int k = 0; k < 3; ++k) { o.a[k] = sxyz[(size_t)i * 3 + k]; o.b[k] = exyz[(size_t)i * 3 + k]; }
   o.a_ref = sref[i]; o.b_ref = eref[i]; o.scene = scene; o.out = i;
+  o.cost_slot = kNoCostSlot; o.pad = 0;
   q[i] = o;
 }
 __global__ void k_random_points(NavData nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref) {
@@ -480,7 +519,9 @@ __global__ void k_random_points(NavData nav, uint32_t scene, const float* u, uin
   oxyz[(size_t)i * 3] = p[0]; oxyz[(size_t)i * 3 + 1] = p[1]; oxyz[(size_t)i * 3 + 2] = p[2];
   oref[i] = ok ? (s.ref_base | ip) : 0;
 }
-__global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
+__global__ void k_set_counts(uint32_t* p, uint32_t n) {
+  if (threadIdx.x <= (uint32_t)kGeoClasses) p[threadIdx.x] = threadIdx.x == 0 ? n : 0u;
+}
 
 }  // namespace
 
@@ -493,9 +534,11 @@ uint32_t geodesic_blocks_per_cu() {
   return (uint32_t)n;
 }
 
-void launch_geodesic(const NavData& nav, const GeoQuery* queries, const uint32_t* count, uint32_t* head, float* out,
-                     GeoSlot* slots, uint32_t num_blocks, uint64_t* counters, hipStream_t st) {
-  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(64), 0, st, nav, queries, count, head, out, slots, counters);
+void launch_geodesic(const NavData& nav, const GeoQuery* queries, uint32_t stride, const uint32_t* counts, uint32_t* head,
+                     float* out, uint32_t* last_cost, GeoSlot* slots, uint32_t num_blocks, uint64_t* counters,
+                     hipStream_t st) {
+  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(64), 0, st, nav, queries, stride, counts, head, out, last_cost,
+                     slots, counters);
 }
 
 void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
@@ -509,7 +552,8 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   mark();
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
   mark();
-  launch_geodesic(nav, Q.queries, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, A.last_cost, slots, geo_blocks,
+                  P.counters, st);
   mark();
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
   mark();
@@ -520,7 +564,8 @@ void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q,
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
   hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
-  launch_geodesic(nav, Q.queries, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, slots, geo_blocks, P.counters, st);
+  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, A.last_cost, slots, geo_blocks,
+                  P.counters, st);
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
 }
 
@@ -533,16 +578,29 @@ void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz
   hipLaunchKernelGGL(k_try_step_batch, grid_for(n, 64), dim3(64), 0, st, nav, scene, sxyz, sref, exyz, n, oxyz, oref);
 }
 void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
-                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [2] */, float* out,
+                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 1] */, float* out,
                            GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st) {
   hipLaunchKernelGGL(k_make_queries, grid_for(n, 256), dim3(256), 0, st, scene, sxyz, sref, exyz, eref, n, qbuf);
-  hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, st, &count_head[0], n);
-  hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, st, &count_head[1], 0u);
-  launch_geodesic(nav, qbuf, &count_head[0], &count_head[1], out, slots, geo_blocks, counters, st);
+  // all in the first class
+  hipLaunchKernelGGL(k_set_counts, dim3(1), dim3(64), 0, st, count_head, n);
+  launch_geodesic(nav, qbuf, n, &count_head[0], &count_head[kGeoClasses], out, nullptr, slots, geo_blocks, counters, st);
 }
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,
                           hipStream_t st) {
   hipLaunchKernelGGL(k_random_points, grid_for(n, 64), dim3(64), 0, st, nav, scene, u, n, oxyz, oref);
 }
 
+#ifdef BPSX_QUERY_TRACE
+extern "C" __attribute__((visibility("default"))) int bpsx_debug_trace(unsigned long long* out, unsigned int max_rows) {
+  unsigned int n = 0;
+  (void)hipDeviceSynchronize();
+  (void)hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_trace_n), 4);
+  if (n > (1u << 17)) n = 1u << 17;
+  if (n > max_rows) n = max_rows;
+  if (out && n) (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), (size_t)n * 32);
+  const unsigned int zero = 0;
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace_n), &zero, 4);
+  return (int)n;
+}
+#endif
 }  // namespace bpsx
