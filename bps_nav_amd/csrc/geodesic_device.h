@@ -265,30 +265,32 @@ struct RegHeap {
     }
     set(q, t, n);
   }
-  // Below 64 entries (almost always) only the first register pair is in use and the walks
-  // need no pair selection.
-  BPSX_DEV void bubble_up_small(int q, uint32_t t, uint32_t n) {
-    while (q > 1) {
-      const int p = q >> 1;
-      const uint32_t pt = rlane(t0, p);
-      if (!(pt > t)) break;
-      const uint32_t pn = rlane(n0, p);
-      t0 = wlane(t0, pt, q);
-      n0 = wlane(n0, pn, q);
-      q = p;
-    }
-    t0 = wlane(t0, t, q);
-    n0 = wlane(n0, n, q);
+  // Below 64 entries (almost always) only the first register pair is in use, and bubbleUp is
+  // done by all lanes at once: the lanes on the way from position q to the root read their
+  // parent's entry; ancestors with a greater key move one step down that way (they form a run
+  // from q upwards, keys never increase towards the root) and the entry lands on top of the run.
+  BPSX_DEV void bubble_up_small(int q, uint32_t t, uint32_t n, int lane) {
+    const int lq = 31 - __clz(q);
+    const int lj = 31 - __clz(lane);            // -1 for lane 0, which is no heap position
+    const int up = lq - lj;                       // levels between this lane's depth and q's
+    const bool on = lane >= 1 && up >= 0 && (q >> (up & 31)) == lane;
+    const uint32_t pk = (uint32_t)__builtin_amdgcn_ds_bpermute((lane >> 1) * 4, (int)t0);
+    const uint32_t pn = (uint32_t)__builtin_amdgcn_ds_bpermute((lane >> 1) * 4, (int)n0);
+    const bool parentMoves = on && lane > 1 && pk > t;
+    const bool vacant = lane == q || t0 > t;
+    const bool land = on && vacant && !parentMoves;
+    t0 = parentMoves ? pk : (land ? t : t0);
+    n0 = parentMoves ? pn : (land ? n : n0);
   }
-  BPSX_DEV void push(uint32_t t, uint32_t n) {
+  BPSX_DEV void push(uint32_t t, uint32_t n, int lane) {
     size++;
-    if (size < 64) bubble_up_small(size, t, n);
+    if (size < 64) bubble_up_small(size, t, n, lane);
     else bubble_up(size, t, n);
   }
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
     if (size < 64) {
       const unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);
-      if (m) bubble_up_small(__ffsll((long long)m) - 1, t, n);
+      if (m) bubble_up_small(__ffsll((long long)m) - 1, t, n, lane);
       return;
     }
     int q = 0;
@@ -536,7 +538,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         else g.push<true>(t, node);
       } else {
         if (open) rh.modify((uint32_t)node, __float_as_uint(t), lane);
-        else rh.push(__float_as_uint(t), (uint32_t)node);
+        else rh.push(__float_as_uint(t), (uint32_t)node, lane);
       }
       if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = node; }
     }
@@ -590,7 +592,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.outOfNodes = false;
     st.expanded = 0;
     st.rh.init();
-    st.rh.push(__float_as_uint(total), 0u);
+    st.rh.push(__float_as_uint(total), 0u, lane);
   }
   AstarExit ex = ASTAR_RUN(0);
   if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
