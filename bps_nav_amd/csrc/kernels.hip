@@ -226,6 +226,9 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         q.cost_slot = done ? kNoCostSlot : gi;   // a finished episode's search predicts nothing
         q.pad = 0;
         cls = geo_class(A.last_cost[gi]);
+        // the first search of an episode ran the other way (agent -> goal) and says little about
+        // the cost of goal -> agent: assume an upper-middle length for the first step
+        if (step <= 2 && cls > 1) cls = 1;
       }
       if (done) {
         // the terminal query above holds copies of the old episode's points: the pose arrays can
@@ -459,7 +462,11 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
       }
 #endif
       out[q.out] = d;
-      if (last_cost && q.cost_slot != kNoCostSlot) last_cost[q.cost_slot] = pops - pops0;
+      // estimate for the agent's next search: this one's length, decaying from earlier peaks
+      if (last_cost && q.cost_slot != kNoCostSlot) {
+        const uint32_t prev = last_cost[q.cost_slot], now = pops - pops0, faded = prev - (prev >> 2);
+        last_cost[q.cost_slot] = now > faded ? now : faded;
+      }
     }
     done++;
     wave_sync();
