@@ -243,10 +243,12 @@ struct GeoWave {
 // are sums of distances, never negative and never NaN, and for such floats the integer order
 // of the bits is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
 constexpr int kRegHeap = 127;
+static_assert(kMaxNodes <= 2048, "heap entries keep the node index in 11 bits");
 static_assert(kHeapLds > kRegHeap, "the register heap must fit the LDS heap it is moved to");
 struct RegHeap {
   uint32_t t0, t1;   // total bits
-  uint32_t n0, n1;   // node index
+  uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11, so that popping
+                     // the root names the edge records to fetch without a detour through LDS
   int size;
 
   BPSX_DEV uint32_t T(int q) const { return q < 64 ? rlane(t0, q) : rlane(t1, q & 63); }
@@ -289,7 +291,7 @@ struct RegHeap {
   }
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
     if (size < 64) {
-      const unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);
+      const unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);   // n: packed like n0
       if (m) bubble_up_small(__ffsll((long long)m) - 1, t, n, lane);
       return;
     }
@@ -400,7 +402,22 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (M == 0 && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
     if (!SH && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
     // the node about to be popped is the root: fetch its edges while the heap is repaired
-    const int bi = SH ? uniform_i((int)L->heap[0].node) : (int)rlane(rh.n0, 1);
+    int bi;
+    uint32_t bestIp;
+    if (SH) {
+      bi = uniform_i((int)L->heap[0].node);
+      bestIp = link_id((uint32_t)uniform_i((int)g.link<S>(bi)));
+    } else {
+      const uint32_t root = rlane(rh.n0, 1);
+      bi = (int)(root & 0x7ffu);
+      bestIp = root >> 11;
+    }
+    uint32_t nb = kNoNb;
+    float m0 = 0, m1 = 0, m2 = 0;
+    if (lane < kNvp) {
+      const AEdge e = edges[bestIp * kNvp + lane];
+      nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
+    }
     float b0, b1, b2, bcost;
     if (g.in_window(bi)) {
       const int w = bi & (kWindow - 1);
@@ -411,14 +428,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
       BPSX_KEEP_APART();
     }
-    const uint32_t bestIp = link_id((uint32_t)uniform_i((int)g.link<S>(bi)));
     const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)g.state<S>(bi)));
-    uint32_t nb = kNoNb;
-    float m0 = 0, m1 = 0, m2 = 0;
-    if (lane < kNvp) {
-      const AEdge e = edges[bestIp * kNvp + lane];
-      nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
-    }
     PHASE_MARK(0);
     if (SH) g.pop<true>();
     else rh.pop(lane);
@@ -526,10 +536,12 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     // ---- ordered phase: heap and "nearest so far" updates in edge order
     unsigned long long upd = __ballot(update);
     const unsigned long long openMask = __ballot(update && wasOpen);
+    const uint32_t packed = (uint32_t)ni | (nb << 11);   // heap entry of this lane's node
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
-      const int node = lane_i(ni, src);
+      const uint32_t entry = rlane(packed, src);
+      const int node = (int)(entry & 0x7ffu);
       const float t = lane_f(total, src);
       const float h = lane_f(heuristic, src);
       const bool open = (openMask >> src) & 1ull;
@@ -537,8 +549,8 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         if (open) g.modify<true>(node, t);
         else g.push<true>(t, node);
       } else {
-        if (open) rh.modify((uint32_t)node, __float_as_uint(t), lane);
-        else rh.push(__float_as_uint(t), (uint32_t)node, lane);
+        if (open) rh.modify(entry, __float_as_uint(t), lane);
+        else rh.push(__float_as_uint(t), entry, lane);
       }
       if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = node; }
     }
@@ -592,7 +604,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.outOfNodes = false;
     st.expanded = 0;
     st.rh.init();
-    st.rh.push(__float_as_uint(total), 0u, lane);
+    st.rh.push(__float_as_uint(total), startIp << 11, lane);
   }
   AstarExit ex = ASTAR_RUN(0);
   if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
@@ -600,8 +612,8 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     g.heapSpills++;
     // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
     const RegHeap& rh = st.rh;
-    if (lane >= 1 && lane <= rh.size) g.L->heap[lane - 1] = HeapEntry{__uint_as_float(rh.t0), rh.n0};
-    if (64 + lane <= rh.size) g.L->heap[63 + lane] = HeapEntry{__uint_as_float(rh.t1), rh.n1};
+    if (lane >= 1 && lane <= rh.size) g.L->heap[lane - 1] = HeapEntry{__uint_as_float(rh.t0), rh.n0 & 0x7ffu};
+    if (64 + lane <= rh.size) g.L->heap[63 + lane] = HeapEntry{__uint_as_float(rh.t1), rh.n1 & 0x7ffu};
     g.heapSize = rh.size;
     wave_sync();
     ex = ASTAR_RUN(2);
