@@ -232,7 +232,7 @@ def test_full_size_workload_properties(oracle, torch_cuda):
         st = {k: v.cpu().numpy() for k, v in gen.get_state(0).items()}
         out = dict(info=gen.get_infos(0).packed.cpu().numpy(), rew=gen.get_rewards(0).cpu().numpy(),
                    polar=gen.get_polars(0).cpu().numpy(), pos=st["position"], ref=st["poly_ref"],
-                   mask=gen.get_masks(0).cpu().numpy())
+                   mask=gen.get_masks(0).cpu().numpy(), goal=st["goal"])
         runs.append(out)
         if rep == 0:
             cnt = gen.counters()
@@ -251,6 +251,12 @@ def test_full_size_workload_properties(oracle, torch_cuda):
         pos = r["pos"][ids]
         x, ref = onav.snap(pos)
         assert np.array_equal(ref, r["ref"][ids].view(np.uint32)), "agents stand where the oracle snaps them"
+        # agents that just moved forward and go on: the distance shown is geodesic(goal point -> agent point)
+        fresh = (acts[-1][ids] == 1) & (r["mask"][ids] == 1)
+        gx, gref = onav.snap(r["goal"][ids])
+        want = onav.geodesic(gx[fresh], gref[fresh], pos[fresh], ref[fresh])
+        assert fresh.sum() > 8
+        assert np.array_equal(common.bits(want), common.bits(r["info"][ids][fresh, 2])), "distance differs from the oracle's"
         onav.close()
     # straight-line bound, all agents: geodesic(goal point -> agent) >= |goal - agent| (3-D), using rho of the polar
     d = r["info"][:, 2]
