@@ -70,6 +70,62 @@ def test_batched_queries_match_oracle(oracle, torch_cuda, config):
     gen.close()
 
 
+@pytest.mark.parametrize("name", ["recast_room", "recast_two_floors"])
+def test_recast_built_meshes_match_reference_vectors(oracle, torch_cuda, name):
+    """Navmeshes built by the reference's own Recast (committed fixtures): the engine against the
+    vectors and simulator traces that the compiled reference wrote for them, and against the
+    oracle on fresh random queries."""
+    import os
+    from bps_nav_amd import scenes
+    from oracle import bpo
+    print(f"case: recast-built fixture {name}", flush=True)
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    with open(os.path.join(gold, name + ".navmesh"), "rb") as f:
+        blob = f.read()
+    g = np.load(os.path.join(gold, name + ".npz"))
+    gen = make_gen([(blob, g["episodes"])], 24, seed=33, max_steps=50)
+    sx, sr = gen.snap_points(0, g["snap_in"])
+    assert np.array_equal(sr, g["snap_ref"]) and np.array_equal(common.bits(sx), common.bits(g["snap_xyz"]))
+    tx, tr = gen.try_steps(0, g["step_start"], g["snap_ref"], g["step_end"])
+    assert np.array_equal(tr, g["step_ref"]) and np.array_equal(common.bits(tx), common.bits(g["step_xyz"]))
+    p = g["geo_perm"]
+    gd = gen.geodesic(0, g["step_start"], g["snap_ref"], g["step_start"][p], g["snap_ref"][p])
+    assert np.array_equal(common.bits(gd), common.bits(g["geo_dist"]))
+    # fresh queries against the oracle
+    nav = bpo.Nav(oracle, blob)
+    rng = np.random.default_rng(9)
+    pts = scenes.sample_points(blob, 13, 1500)
+    q = pts + rng.normal(0, 0.3, pts.shape).astype(np.float32)
+    q[:, 1] += rng.uniform(-1, 2, len(q)).astype(np.float32)
+    xo, ro = nav.snap(q)
+    xg, rg = gen.snap_points(0, q)
+    assert np.array_equal(ro, rg) and np.array_equal(common.bits(xo), common.bits(xg))
+    gen.close()
+    for mode in (0, 1):
+        gen = make_gen([(blob, g["episodes"])], 24, seed=33, max_steps=50, reset_mode=mode)
+        gen.reset(0)
+        state, infos = gen.get_state(0), gen.get_infos(0)
+        assert np.array_equal(state["poly_ref"].cpu().numpy().view(np.uint32), g[f"sim{mode}_reset_poly_ref"])
+        for t, a in enumerate(g[f"sim{mode}_actions"]):
+            gen.step(0, a)
+            st = {k: v.cpu().numpy() for k, v in state.items()}
+            for k in ("poly_ref", "goal_ref", "step", "episode", "num_resets"):
+                assert np.array_equal(st[k].view(np.uint32), g[f"sim{mode}_{k}"][t]), f"{k} at step {t} mode {mode}"
+            assert np.array_equal(common.bits(st["position"]), common.bits(g[f"sim{mode}_position"][t]))
+            assert np.array_equal(gen.get_masks(0).cpu().numpy(), g[f"sim{mode}_masks"][t])
+            gi = infos.packed.cpu().numpy()
+            assert np.array_equal(common.bits(gi), common.bits(g[f"sim{mode}_infos"][t])) or np.isnan(gi).any(), f"infos at step {t}"
+            np.testing.assert_allclose(gi, g[f"sim{mode}_infos"][t], rtol=1e-3, equal_nan=True)
+            np.testing.assert_allclose(gen.get_rewards(0).cpu().numpy(), g[f"sim{mode}_rewards"][t], rtol=1e-3, atol=1e-6,
+                                       equal_nan=True)
+            gp, cp = gen.get_polars(0).cpu().numpy(), g[f"sim{mode}_polars"][t]
+            np.testing.assert_allclose(gp[:, 0], cp[:, 0], rtol=1e-6, atol=1e-6)
+            dphi = np.abs(gp[:, 1] - cp[:, 1])
+            assert (np.minimum(dphi, 2 * np.pi - dphi) < 1e-4).all()
+        gen.check_errors()
+        gen.close()
+
+
 def test_open_hall_queries_match_oracle(oracle, torch_cuda):
     """A hall without obstacles: A* spreads over a wide front, so the open list outgrows the
     kernel's register heap, the node links outgrow LDS and long queries exhaust Detour's

@@ -72,6 +72,40 @@ def test_simulator_traces(oracle, path):
     assert (g["masks"] == 0).sum() > 0
 
 
+RECAST_FIXTURES = ("recast_room", "recast_two_floors")
+
+
+def load_recast(name):
+    with open(os.path.join(GOLD, name + ".navmesh"), "rb") as f:
+        return f.read(), np.load(os.path.join(GOLD, name + ".npz"))
+
+
+@pytest.mark.parametrize("name", RECAST_FIXTURES)
+def test_recast_built_mesh_queries_and_traces(oracle, name):
+    """Navmeshes made by the reference's own Recast (irregular polygons, detail meshes with extra
+    height samples, islands on obstacles; two floors overlapping in xz joined by a ramp): queries
+    and whole simulator traces of the compiled reference, bit for bit."""
+    blob, g = load_recast(name)
+    nav = bpo.Nav(oracle, blob)
+    gd = check_queries(nav, g)
+    assert np.isinf(gd).any() and np.isfinite(gd).any()       # box tops / unreachable parts are islands
+    if name == "recast_two_floors":
+        y = g["snap_xyz"][:, 1]
+        assert (y[np.isfinite(y)] < 0.5).any() and (y[np.isfinite(y)] > 2.0).any()   # both floors are hit
+    for mode in (0, 1):
+        sim = bpo.Sim(oracle, [(blob, g["episodes"])], 24, reset_mode=mode, seed=33, max_steps=50, threads=2)
+        sim.reset()
+        assert np.array_equal(sim.state()["poly_ref"], g[f"sim{mode}_reset_poly_ref"])
+        for t, a in enumerate(g[f"sim{mode}_actions"]):
+            sim.step(a)
+            o, s = sim.outputs(), sim.state()
+            for k in ("rewards", "masks", "infos", "polars"):
+                assert np.array_equal(o[k], g[f"sim{mode}_{k}"][t], equal_nan=True), f"{k} differs at step {t} (mode {mode})"
+            for k in ("position", "rotation", "poly_ref", "goal_ref", "step", "episode", "num_resets"):
+                assert np.array_equal(s[k], g[f"sim{mode}_{k}"][t], equal_nan=True), f"{k} differs at step {t} (mode {mode})"
+        assert (g[f"sim{mode}_masks"] == 0).sum() > 0
+
+
 def test_random_point_in_convex_poly_golden(oracle):
     g = np.load(os.path.join(GOLD, "random_point.npz"))
     for row, (s, t), want in zip(g["polys"], g["st"], g["out"]):
