@@ -159,12 +159,16 @@ constexpr uint32_t kNoCostSlot = 0xffffffffu;
 
 // Path searches differ in length by two orders of magnitude and each is sequential, so a step
 // ends when its longest search ends.  Queries are therefore queued in classes of expected
-// cost (the nodes the agent's previous search expanded) and the longest class is served
-// first; a search that runs long also raises its wavefront's issue priority.
-constexpr int kGeoClasses = 4;
-inline __host__ __device__ uint32_t geo_class(uint32_t last_cost) {
-  return last_cost >= 1024u ? 0u : last_cost >= 512u ? 1u : last_cost >= 192u ? 2u : 3u;
+// cost (the nodes the agent's previous searches expanded) and served from the longest class
+// down, which approximates longest-first scheduling; a search that runs long also raises its
+// wavefront's issue priority.
+constexpr int kGeoClasses = 16;
+constexpr uint32_t kGeoClassWidth = 100;   // expanded nodes per class: 1500 and more, 1400-1499, ..., below 100
+constexpr __host__ __device__ uint32_t geo_class(uint32_t last_cost) {
+  return last_cost / kGeoClassWidth >= (uint32_t)kGeoClasses ? 0u
+                                                             : (uint32_t)kGeoClasses - 1u - last_cost / kGeoClassWidth;
 }
+constexpr uint32_t kGeoClassUnknown = geo_class(700);   // a search without history: upper-middle length
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,

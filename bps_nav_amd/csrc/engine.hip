@@ -237,7 +237,7 @@ int bpsx_finalize(bpsx_sim* sim) {
   sim->groups.resize(sim->num_groups);
   const size_t n = sim->envs_per_group;
   for (auto& g : sim->groups) {
-    if ((rc = sim->alloc(&g.Q.counts, 8)) || (rc = sim->alloc(&g.Q.queries, (size_t)kGeoClasses * 2 * n)) ||
+    if ((rc = sim->alloc(&g.Q.counts, kGeoClasses + 2)) || (rc = sim->alloc(&g.Q.queries, (size_t)kGeoClasses * 2 * n)) ||
         (rc = sim->alloc(&g.Q.reset_list, n)) || (rc = sim->alloc(&g.d_actions, n)))
       return rc;
     g.Q.stride = (uint32_t)(2 * n);

@@ -10,7 +10,7 @@ enum QueueCounter { kQGeo = 0 /* one per cost class */, kQGeoHead = kGeoClasses,
 
 // Work queues of one step, all in HBM, sized for every agent of a group.
 struct StepQueues {
-  uint32_t* counts;          // [8], see QueueCounter
+  uint32_t* counts;          // [kGeoClasses + 2], see QueueCounter
   GeoQuery* queries;         // [kGeoClasses][stride]: one per moved/finished agent plus one per reset
   uint32_t stride;           // 2n
   uint32_t* reset_list;      // [n] agent indices being reset

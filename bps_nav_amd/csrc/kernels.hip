@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         cls = geo_class(A.last_cost[gi]);
         // the first search of an episode ran the other way (agent -> goal) and says little about
         // the cost of goal -> agent: assume an upper-middle length for the first step
-        if (step <= 2 && cls > 1) cls = 1;
+        if (step <= 2 && cls > kGeoClassUnknown) cls = kGeoClassUnknown;
       }
       if (done) {
         // the terminal query above holds copies of the old episode's points: the pose arrays can
@@ -238,11 +238,7 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
       }
     }
   }
-  for (uint32_t c = 0; c < (uint32_t)kGeoClasses; ++c) {
-    const bool mine = want && cls == c;
-    const uint32_t slot = wave_append(mine, &Q.counts[kQGeo + c]);
-    if (mine) Q.queries[(size_t)c * Q.stride + slot] = q;
-  }
+  if (want) Q.queries[(size_t)cls * Q.stride + atomicAdd(&Q.counts[kQGeo + cls], 1u)] = q;
   const uint32_t rslot = wave_append(reset, &Q.counts[kQReset]);
   if (reset) Q.reset_list[rslot] = gi;
   // counters, one atomic per wavefront
@@ -401,8 +397,8 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
       q.out = P.total + gi;
       q.cost_slot = gi;
       q.pad = 0;
-      // a new episode: no history, assume a search of upper-middle length
-      Q.queries[(size_t)1 * Q.stride + atomicAdd(&Q.counts[kQGeo + 1], 1u)] = q;
+      // a new episode: no history
+      Q.queries[(size_t)kGeoClassUnknown * Q.stride + atomicAdd(&Q.counts[kQGeo + kGeoClassUnknown], 1u)] = q;
     }
   }
   if (lane == 0 && blockIdx.x == 0 && n) atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
@@ -445,8 +441,9 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
     const uint32_t pops0 = pops;
 #ifdef BPSX_QUERY_TRACE
     const unsigned long long trace_t0 = wall_clock64();
+    const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
-    g.basePrio = kGeoClasses - 1 - cls;
+    g.basePrio = (kGeoClasses - 1 - cls) >> 2;
     set_wave_priority(g.basePrio);
 #ifdef BPSX_PHASE_TIMING
     const float d = geodesic_query(g, nav, q, &pops, &corridor, phase_acc);
@@ -458,7 +455,7 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
       const unsigned int ti = atomicAdd(&g_trace_n, 1u);
       if (ti < (1u << 17)) {
         g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = pops - pops0;
-        g_trace[ti][3] = (unsigned long long)cls | ((unsigned long long)blockIdx.x << 8) | ((unsigned long long)qi << 32);
+        g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)qi << 32);
       }
 #endif
       out[q.out] = d;
