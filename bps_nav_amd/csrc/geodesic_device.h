@@ -121,6 +121,9 @@ struct GeoWave {
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
   int basePrio;                      // issue priority the query started with
+#ifdef BPSX_QUERY_TRACE
+  uint32_t missTop, missNb, maxHeap;
+#endif
 
   // ---------------------------------------------------------------- node pool
   template <bool S> BPSX_DEV uint32_t link(int i) const {
@@ -398,7 +401,13 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
       b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
       BPSX_KEEP_APART();
+#ifdef BPSX_QUERY_TRACE
+      g.missTop++;
+#endif
     }
+#ifdef BPSX_QUERY_TRACE
+    if (!SH && (uint32_t)rh.size > g.maxHeap) g.maxHeap = (uint32_t)rh.size;
+#endif
     const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)g.state<S>(bi)));
     PHASE_MARK(0);
     if (SH) g.pop<true>();
@@ -455,12 +464,16 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       }
     }
     PHASE_MARK(4);
+#ifdef BPSX_QUERY_TRACE
+    g.missNb += (uint32_t)__popcll(__ballot(nb != kNoNb && !isNew && !g.in_window(ni)));
+#endif
     bool update = false, wasOpen = false;
     float total = 0, heuristic = 0;
     if (nb != kNoNb) {
       float p0 = m0, p1 = m1, p2 = m2, oldTotal = 0;
       uint32_t fl = 0;
       const bool inw = g.in_window(ni);   // new nodes always are
+
       const int w = ni & (kWindow - 1);
       ANode& hn = g.ws->nodes[ni];
       if (!isNew) {

@@ -441,6 +441,7 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
     const uint32_t pops0 = pops;
 #ifdef BPSX_QUERY_TRACE
     const unsigned long long trace_t0 = wall_clock64();
+    g.missTop = g.missNb = g.maxHeap = 0;
     const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
     g.basePrio = (kGeoClasses - 1 - cls) >> 2;
@@ -455,7 +456,8 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
       const unsigned int ti = atomicAdd(&g_trace_n, 1u);
       if (ti < (1u << 17)) {
         g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = pops - pops0;
-        g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)qi << 32);
+        g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)(g.missTop & 0xfffu) << 24) |
+                          ((unsigned long long)(g.missNb & 0xfffu) << 36) | ((unsigned long long)(g.maxHeap & 0xffu) << 48);
       }
 #endif
       out[q.out] = d;
