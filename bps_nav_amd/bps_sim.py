@@ -73,7 +73,7 @@ class PointNavRolloutGenerator:
 
     def __init__(self, dataset_path, asset_path, num_environments, num_active_scenes, num_workers=-1, gpu_id=0,
                  render_resolution=(64, 64), color=False, depth=False, double_buffered=False, seed=0,
-                 should_set_affinity=True, *, scenes=None, reset_mode=0, max_steps=0):
+                 should_set_affinity=True, *, scenes=None, reset_mode=0, max_steps=0, scene_reserve=0.0):
         self._L = _lib.lib()
         if not hasattr(self._L, "bpsx_create"):
             raise RuntimeError("libbpsx.so was built without the HIP engine")
@@ -87,7 +87,7 @@ class PointNavRolloutGenerator:
         self.gpu_id = gpu_id
         self.double_buffered = bool(double_buffered)
         cfg = _lib.Config(num_environments, num_active_scenes, int(self.double_buffered), reset_mode, seed, gpu_id,
-                          max_steps, self.TASK)
+                          max_steps, self.TASK, scene_reserve)
         h = C.c_void_p()
         _lib.check(self._L.bpsx_create(C.byref(cfg), C.byref(h)))
         self._h = h
@@ -186,9 +186,11 @@ class PointNavRolloutGenerator:
 
     @property
     def swap_stats(self):
-        """(swap fraction, scenes in use, envs per scene) like simulator.cpp:1412-1424; scenes
-        never rotate here."""
-        return (0.0, float(self.num_scenes), float(self.envs_per_group * self.num_groups) / self.num_scenes)
+        """(scene swaps completed per 100 steps taken, scenes in use, envs per scene) like
+        simulator.cpp:1412-1424."""
+        done = self.swap_status(0)[1]
+        steps = max(1, self.counters()["agent_steps"] // max(1, self.envs_per_group))
+        return (100.0 * done / steps, float(self.num_scenes), float(self.envs_per_group * self.num_groups) / self.num_scenes)
 
     # ---- state and diagnostics for parity harnesses
     def get_state(self, group_idx):
@@ -201,6 +203,21 @@ class PointNavRolloutGenerator:
                     rotation=t(s.rotation, (n, 4), torch.float32, d, self),
                     goal=t(s.goal, (n, 3), torch.float32, d, self), poly_ref=i32(s.poly_ref),
                     goal_ref=i32(s.goal_ref), step=i32(s.step), episode=i32(s.episode), num_resets=i32(s.num_resets))
+
+    # ---- scene rotation
+    def swap_scene(self, slot, navmesh_bytes, episodes):
+        """Starts replacing the scene of slot `slot`: each of its envs moves to the new scene when
+        its episode ends (SceneSwapper, simulator.cpp:1063-1154).  RuntimeError while the slot's
+        previous swap is still in progress."""
+        eps = np.ascontiguousarray(episodes, np.float32).reshape(-1, 10)
+        _lib.check(self._L.bpsx_swap_scene(self._h, slot, navmesh_bytes, len(navmesh_bytes),
+                                           eps.ctypes.data if len(eps) else None, len(eps)))
+
+    def swap_status(self, slot):
+        """(envs of the slot still on the old scene, swaps completed since creation)"""
+        rem, done = C.c_uint32(), C.c_uint64()
+        _lib.check(self._L.bpsx_swap_status(self._h, slot, C.byref(rem), C.byref(done)))
+        return rem.value, done.value
 
     def check_errors(self):
         _lib.check(self._L.bpsx_check_errors(self._h))

@@ -46,6 +46,51 @@ int dev_alloc(T** p, size_t count) {
 
 }  // namespace
 
+// First-fit allocator over one of the concatenated navmesh arrays (units = elements).  Scenes
+// come and go with scene rotation; neighbouring free ranges are merged on release.
+struct Arena {
+  size_t cap = 0;
+  std::vector<std::pair<size_t, size_t>> free_ranges;   // (offset, length), sorted by offset
+  void init(size_t capacity) { cap = capacity; free_ranges.assign(1, {0, capacity}); }
+  bool take(size_t len, size_t* off) {
+    if (len == 0) { *off = 0; return true; }
+    for (size_t i = 0; i < free_ranges.size(); ++i) {
+      if (free_ranges[i].second < len) continue;
+      *off = free_ranges[i].first;
+      free_ranges[i].first += len;
+      free_ranges[i].second -= len;
+      if (!free_ranges[i].second) free_ranges.erase(free_ranges.begin() + (long)i);
+      return true;
+    }
+    return false;
+  }
+  void give(size_t off, size_t len) {
+    if (!len) return;
+    size_t i = 0;
+    while (i < free_ranges.size() && free_ranges[i].first < off) ++i;
+    free_ranges.insert(free_ranges.begin() + (long)i, {off, len});
+    for (size_t k = 0; k + 1 < free_ranges.size();) {
+      if (free_ranges[k].first + free_ranges[k].second == free_ranges[k + 1].first) {
+        free_ranges[k].second += free_ranges[k + 1].second;
+        free_ranges.erase(free_ranges.begin() + (long)k + 1);
+      } else {
+        ++k;
+      }
+    }
+  }
+};
+// Where one resident scene lives in the arrays.
+struct SceneRanges {
+  size_t poly = 0, npoly = 0, bv = 0, nbv = 0, tri = 0, ntri = 0, dv = 0, ndv = 0, ep = 0, nep = 0;
+  bool used = false;
+};
+// A scene slot has two scene-table entries (slot and slot + num_active_scenes): the scene its
+// envs are on and, during a swap, the scene they are moving to.
+struct SceneSlot {
+  uint32_t current = 0;         // scene-table entry of the resident scene
+  uint32_t target = kNoSwap;    // entry of the scene being moved to, if a swap is in progress or just done
+};
+
 struct bpsx_sim {
   bpsx_config cfg{};
   std::vector<HostScene> scenes;
@@ -60,6 +105,12 @@ struct bpsx_sim {
   SceneDev* d_scenes = nullptr;
   float* d_episodes = nullptr;
   NavData nav{};
+  Arena ar_poly, ar_bv, ar_tri, ar_dv, ar_ep;
+  std::vector<SceneRanges> ranges;   // per scene-table entry
+  std::vector<SceneSlot> slots;
+  uint32_t* d_swap_target = nullptr;
+  uint32_t* d_swap_remaining = nullptr;
+  uint64_t swaps_completed = 0;
   AgentArrays A{};
   std::vector<void*> owned;  // every device allocation, for destroy
   std::vector<Group> groups;
@@ -98,6 +149,9 @@ struct bpsx_sim {
     memcpy(P.turn_right, turn_right, 16);
     P.error_flag = d_error;
     P.counters = d_counters;
+    P.num_slots = cfg.num_active_scenes;
+    P.swap_target = d_swap_target;
+    P.swap_remaining = d_swap_remaining;
     return P;
   }
 };
@@ -147,49 +201,89 @@ int bpsx_add_scene(bpsx_sim* sim, const void* navmesh_bytes, size_t navmesh_size
   return BPSX_OK;
 }
 
+// Places one parsed scene into the arrays and writes its scene-table entry.
+static int upload_scene(bpsx_sim* sim, HostScene& s, uint32_t entry) {
+  SceneRanges r;
+  r.npoly = s.polys.size(); r.nbv = s.bv.size(); r.ntri = s.dtris.size() / 4; r.ndv = s.dverts.size() / 3;
+  r.nep = s.episodes.size() / 10;
+  const bool a = sim->ar_poly.take(r.npoly, &r.poly);
+  const bool b = a && sim->ar_bv.take(r.nbv, &r.bv);
+  const bool c = b && sim->ar_tri.take(r.ntri, &r.tri);
+  const bool d = c && sim->ar_dv.take(r.ndv, &r.dv);
+  const bool e = d && sim->ar_ep.take(r.nep, &r.ep);
+  if (!e) {
+    if (a) sim->ar_poly.give(r.poly, r.npoly);
+    if (b) sim->ar_bv.give(r.bv, r.nbv);
+    if (c) sim->ar_tri.give(r.tri, r.ntri);
+    if (d) sim->ar_dv.give(r.dv, r.ndv);
+    return fail(BPSX_E_UNSUPPORTED, "scene does not fit the space reserved for scene rotation");
+  }
+  r.used = true;
+  s.dev.poly_base = (uint32_t)r.poly; s.dev.bv_base = (uint32_t)r.bv; s.dev.ep_base = (uint32_t)r.ep;
+  s.dev.ep_count = (uint32_t)r.nep;
+  for (auto& p : s.polys) { p.tri_base += (uint32_t)r.tri; p.dvert_base += (uint32_t)r.dv; }
+  HIP_TRY(hipMemcpy(sim->d_polys + r.poly, s.polys.data(), r.npoly * sizeof(PolyRec), hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(sim->d_aedges + r.poly * kNvp, s.aedges.data(), s.aedges.size() * sizeof(AEdge), hipMemcpyHostToDevice));
+  if (r.nbv) HIP_TRY(hipMemcpy(sim->d_bv + r.bv, s.bv.data(), r.nbv * sizeof(BVNodeDev), hipMemcpyHostToDevice));
+  if (r.ntri) HIP_TRY(hipMemcpy(sim->d_dtris + r.tri * 4, s.dtris.data(), s.dtris.size(), hipMemcpyHostToDevice));
+  if (r.ndv) HIP_TRY(hipMemcpy(sim->d_dverts + r.dv * 3, s.dverts.data(), s.dverts.size() * 4, hipMemcpyHostToDevice));
+  if (r.nep) HIP_TRY(hipMemcpy(sim->d_episodes + r.ep * 10, s.episodes.data(), s.episodes.size() * 4, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(sim->d_scenes + entry, &s.dev, sizeof(SceneDev), hipMemcpyHostToDevice));
+  sim->ranges[entry] = r;
+  return BPSX_OK;
+}
+static void release_scene(bpsx_sim* sim, uint32_t entry) {
+  SceneRanges& r = sim->ranges[entry];
+  if (!r.used) return;
+  sim->ar_poly.give(r.poly, r.npoly); sim->ar_bv.give(r.bv, r.nbv); sim->ar_tri.give(r.tri, r.ntri);
+  sim->ar_dv.give(r.dv, r.ndv); sim->ar_ep.give(r.ep, r.nep);
+  r = SceneRanges{};
+}
+
 int bpsx_finalize(bpsx_sim* sim) {
   if (!sim) return fail(BPSX_E_INVAL, "finalize: null simulator");
   if (sim->finalized) return fail(BPSX_E_STATE, "finalize: called twice");
   if (sim->scenes.size() != sim->cfg.num_active_scenes)
     return fail(BPSX_E_INVAL, "finalize: number of scenes added differs from num_active_scenes");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
-  // ---- concatenate scenes
-  size_t npoly = 0, nbv = 0, ntri = 0, ndv = 0, nep = 0;
+  // ---- navmesh arrays: every scene is a range of each array; room for scene rotation
+  size_t npoly = 0, nbv = 0, ntri = 0, ndv = 0, nep = 0, mpoly = 0, mbv = 0, mtri = 0, mdv = 0, mep = 0;
   for (auto& s : sim->scenes) {
-    s.dev.poly_base = (uint32_t)npoly; s.dev.bv_base = (uint32_t)nbv; s.dev.ep_base = (uint32_t)nep;
-    for (auto& p : s.polys) { p.tri_base += (uint32_t)ntri; p.dvert_base += (uint32_t)ndv; }
     npoly += s.polys.size(); nbv += s.bv.size(); ntri += s.dtris.size() / 4; ndv += s.dverts.size() / 3;
     nep += s.episodes.size() / 10;
+    mpoly = std::max(mpoly, s.polys.size()); mbv = std::max(mbv, s.bv.size()); mtri = std::max(mtri, s.dtris.size() / 4);
+    mdv = std::max(mdv, s.dverts.size() / 3); mep = std::max(mep, s.episodes.size() / 10);
   }
-  if (npoly > 0xfffffff0ull || ntri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
+  const double k = sim->cfg.scene_reserve > 0 ? (double)sim->cfg.scene_reserve : 3.0;
+  if (k < 1.0) return fail(BPSX_E_INVAL, "finalize: scene_reserve must be at least 1");
+  auto room = [k](size_t total, size_t largest) { return (size_t)((double)total * k) + largest + 64; };
+  const size_t cpoly = room(npoly, mpoly), cbv = room(nbv, mbv), ctri = room(ntri, mtri), cdv = room(ndv, mdv),
+               cep = room(nep, mep);
+  if (cpoly > 0xfffffff0ull || ctri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
   int rc;
-  if ((rc = sim->alloc(&sim->d_polys, npoly))) return rc;
-  if ((rc = sim->alloc(&sim->d_aedges, npoly * kNvp))) return rc;
-  if ((rc = sim->alloc(&sim->d_bv, nbv))) return rc;
-  if ((rc = sim->alloc(&sim->d_dtris, ntri * 4))) return rc;
-  if ((rc = sim->alloc(&sim->d_dverts, ndv * 3))) return rc;
-  if ((rc = sim->alloc(&sim->d_scenes, sim->scenes.size()))) return rc;
-  if ((rc = sim->alloc(&sim->d_episodes, nep * 10))) return rc;
-  std::vector<SceneDev> sd;
-  for (auto& s : sim->scenes) {
-    HIP_TRY(hipMemcpy(sim->d_polys + s.dev.poly_base, s.polys.data(), s.polys.size() * sizeof(PolyRec), hipMemcpyHostToDevice));
-    HIP_TRY(hipMemcpy(sim->d_aedges + (size_t)s.dev.poly_base * kNvp, s.aedges.data(), s.aedges.size() * sizeof(AEdge), hipMemcpyHostToDevice));
-    if (!s.bv.empty())
-      HIP_TRY(hipMemcpy(sim->d_bv + s.dev.bv_base, s.bv.data(), s.bv.size() * sizeof(BVNodeDev), hipMemcpyHostToDevice));
-    sd.push_back(s.dev);
-  }
-  // detail arrays and episodes are copied with running offsets
-  {
-    size_t toff = 0, voff = 0, eoff = 0;
-    for (auto& s : sim->scenes) {
-      if (!s.dtris.empty()) HIP_TRY(hipMemcpy(sim->d_dtris + toff, s.dtris.data(), s.dtris.size(), hipMemcpyHostToDevice));
-      if (!s.dverts.empty()) HIP_TRY(hipMemcpy(sim->d_dverts + voff, s.dverts.data(), s.dverts.size() * 4, hipMemcpyHostToDevice));
-      if (!s.episodes.empty()) HIP_TRY(hipMemcpy(sim->d_episodes + eoff, s.episodes.data(), s.episodes.size() * 4, hipMemcpyHostToDevice));
-      toff += s.dtris.size(); voff += s.dverts.size(); eoff += s.episodes.size();
-    }
-  }
-  HIP_TRY(hipMemcpy(sim->d_scenes, sd.data(), sd.size() * sizeof(SceneDev), hipMemcpyHostToDevice));
+  const uint32_t S = sim->cfg.num_active_scenes;
+  if ((rc = sim->alloc(&sim->d_polys, cpoly))) return rc;
+  if ((rc = sim->alloc(&sim->d_aedges, cpoly * kNvp))) return rc;
+  if ((rc = sim->alloc(&sim->d_bv, cbv))) return rc;
+  if ((rc = sim->alloc(&sim->d_dtris, ctri * 4))) return rc;
+  if ((rc = sim->alloc(&sim->d_dverts, cdv * 3))) return rc;
+  if ((rc = sim->alloc(&sim->d_scenes, 2 * (size_t)S))) return rc;
+  if ((rc = sim->alloc(&sim->d_episodes, cep * 10))) return rc;
+  if ((rc = sim->alloc(&sim->d_swap_target, S)) || (rc = sim->alloc(&sim->d_swap_remaining, S))) return rc;
+  sim->ar_poly.init(cpoly); sim->ar_bv.init(cbv); sim->ar_tri.init(ctri); sim->ar_dv.init(cdv); sim->ar_ep.init(cep);
+  sim->ranges.assign(2 * (size_t)S, SceneRanges{});
+  sim->slots.assign(S, SceneSlot{});
   sim->nav = NavData{sim->d_polys, sim->d_aedges, sim->d_bv, sim->d_dtris, sim->d_dverts, sim->d_scenes, sim->d_episodes};
+  {
+    std::vector<uint32_t> none(S, kNoSwap);
+    HIP_TRY(hipMemcpy(sim->d_swap_target, none.data(), (size_t)S * 4, hipMemcpyHostToDevice));
+  }
+  for (uint32_t i = 0; i < S; ++i) {
+    sim->slots[i].current = i;
+    if ((rc = upload_scene(sim, sim->scenes[i], i))) return rc;
+  }
+  sim->scenes.clear();   // the host copies are not needed any more
+  sim->scenes.shrink_to_fit();
 
   // ---- agent state
   const size_t N = sim->cfg.num_environments;
@@ -410,9 +504,79 @@ static int batch_reserve(bpsx_sim* sim, size_t bytes) {
   sim->batch_bytes = bytes;
   return BPSX_OK;
 }
+// Brings the host's view of a slot up to date: a swap whose envs have all moved is complete.
+static int settle_slot(bpsx_sim* sim, uint32_t slot, uint32_t* remaining_out) {
+  SceneSlot& sl = sim->slots[slot];
+  uint32_t remaining = 0;
+  if (sl.target != kNoSwap) {
+    HIP_TRY(hipMemcpy(&remaining, sim->d_swap_remaining + slot, 4, hipMemcpyDeviceToHost));
+    if (remaining == 0) {
+      // every env is on the new scene: the old one leaves, the slot has no swap any more
+      release_scene(sim, sl.current);
+      sl.current = sl.target;
+      sl.target = kNoSwap;
+      const uint32_t none = kNoSwap;
+      HIP_TRY(hipMemcpy(sim->d_swap_target + slot, &none, 4, hipMemcpyHostToDevice));
+      sim->swaps_completed++;
+    }
+  }
+  if (remaining_out) *remaining_out = remaining;
+  return BPSX_OK;
+}
+
+int bpsx_swap_scene(bpsx_sim* sim, uint32_t slot, const void* navmesh_bytes, size_t navmesh_size, const float* episodes,
+                    uint32_t num_episodes) {
+  if (!sim || !sim->finalized) return fail(BPSX_E_STATE, "swap_scene: simulator not finalized");
+  if (slot >= sim->cfg.num_active_scenes) return fail(BPSX_E_INVAL, "swap_scene: slot out of range");
+  if (!navmesh_bytes) return fail(BPSX_E_INVAL, "swap_scene: null navmesh");
+  if (sim->cfg.reset_mode == BPSX_RESET_EPISODES && (!episodes || !num_episodes))
+    return fail(BPSX_E_INVAL, "swap_scene: episode-table reset needs at least one episode");
+  for (auto& g : sim->groups)
+    if (g.in_flight) return fail(BPSX_E_STATE, "swap_scene: a step is in flight");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  HIP_TRY(hipDeviceSynchronize());   // nothing may still read a scene that is about to leave
+  uint32_t remaining = 0;
+  int rc = settle_slot(sim, slot, &remaining);
+  if (rc) return rc;
+  if (remaining) return fail(BPSX_E_STATE, "swap_scene: the previous swap of this slot is still in progress");
+  HostScene hs;
+  if ((rc = parse_navmesh((const uint8_t*)navmesh_bytes, navmesh_size, &hs))) return rc;
+  if (episodes && num_episodes) hs.episodes.assign(episodes, episodes + (size_t)num_episodes * 10);
+  SceneSlot& sl = sim->slots[slot];
+  const uint32_t S = sim->cfg.num_active_scenes;
+  const uint32_t entry = sl.current < S ? slot + S : slot;   // the slot's other table entry
+  if ((rc = upload_scene(sim, hs, entry))) return rc;
+  const uint32_t per = sim->cfg.num_environments / S;
+  HIP_TRY(hipMemcpy(sim->d_swap_remaining + slot, &per, 4, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(sim->d_swap_target + slot, &entry, 4, hipMemcpyHostToDevice));
+  sl.target = entry;
+  return BPSX_OK;
+}
+
+int bpsx_swap_status(bpsx_sim* sim, uint32_t slot, uint32_t* envs_remaining, uint64_t* swaps_completed) {
+  if (!sim || !sim->finalized) return fail(BPSX_E_STATE, "swap_status: simulator not finalized");
+  if (slot >= sim->cfg.num_active_scenes) return fail(BPSX_E_INVAL, "swap_status: slot out of range");
+  for (auto& g : sim->groups)
+    if (g.in_flight) return fail(BPSX_E_STATE, "swap_status: a step is in flight");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  HIP_TRY(hipDeviceSynchronize());
+  uint32_t remaining = 0;
+  const int rc = settle_slot(sim, slot, &remaining);
+  if (rc) return rc;
+  if (envs_remaining) *envs_remaining = remaining;
+  if (swaps_completed) *swaps_completed = sim->swaps_completed;
+  return BPSX_OK;
+}
+
+// Batched queries name a scene slot: they see the newest scene uploaded for it.
+static uint32_t scene_entry(const bpsx_sim* sim, uint32_t slot) {
+  const SceneSlot& sl = sim->slots[slot];
+  return sl.target != kNoSwap ? sl.target : sl.current;
+}
+
 static int check_scene(bpsx_sim* sim, uint32_t scene, const char* what) {
   if (!sim || !sim->finalized) return fail(BPSX_E_STATE, std::string(what) + ": simulator not finalized");
-  if (scene >= sim->scenes.size()) return fail(BPSX_E_INVAL, std::string(what) + ": scene out of range");
+  if (scene >= sim->cfg.num_active_scenes) return fail(BPSX_E_INVAL, std::string(what) + ": scene out of range");
   for (auto& g : sim->groups)
     if (g.in_flight) return fail(BPSX_E_STATE, std::string(what) + ": a step is in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
@@ -429,7 +593,7 @@ int bpsx_snap_points(bpsx_sim* sim, uint32_t scene, const float* pts, uint32_t n
   char* b = (char*)sim->d_batch;
   float* d_in = (float*)b; float* d_xyz = (float*)(b + f3); uint32_t* d_ref = (uint32_t*)(b + 2 * f3);
   HIP_TRY(hipMemcpy(d_in, pts, f3, hipMemcpyHostToDevice));
-  launch_snap_batch(sim->nav, scene, d_in, n, d_xyz, d_ref, sim->snap_blocks * 4, nullptr);
+  launch_snap_batch(sim->nav, scene_entry(sim, scene), d_in, n, d_xyz, d_ref, sim->snap_blocks * 4, nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipMemcpy(out_xyz, d_xyz, f3, hipMemcpyDeviceToHost));
   HIP_TRY(hipMemcpy(out_ref, d_ref, (size_t)n * 4, hipMemcpyDeviceToHost));
@@ -450,7 +614,7 @@ int bpsx_try_steps(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const 
   HIP_TRY(hipMemcpy(d_s, start_xyz, f3, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d_e, end_xyz, f3, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d_sr, start_ref, u1, hipMemcpyHostToDevice));
-  launch_try_step_batch(sim->nav, scene, d_s, d_sr, d_e, n, d_o, d_or, nullptr);
+  launch_try_step_batch(sim->nav, scene_entry(sim, scene), d_s, d_sr, d_e, n, d_o, d_or, nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipMemcpy(out_xyz, d_o, f3, hipMemcpyDeviceToHost));
   HIP_TRY(hipMemcpy(out_ref, d_or, u1, hipMemcpyDeviceToHost));
@@ -474,7 +638,7 @@ int bpsx_geodesic(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const u
   HIP_TRY(hipMemcpy(d_e, end_xyz, f3, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d_sr, start_ref, u1, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(d_er, end_ref, u1, hipMemcpyHostToDevice));
-  launch_geodesic_batch(sim->nav, scene, d_s, d_sr, d_e, d_er, n, d_q, sim->d_batch_counts, d_o, sim->d_slots,
+  launch_geodesic_batch(sim->nav, scene_entry(sim, scene), d_s, d_sr, d_e, d_er, n, d_q, sim->d_batch_counts, d_o, sim->d_slots,
                         sim->geo_blocks, sim->d_counters, nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipMemcpy(out_dist, d_o, u1, hipMemcpyDeviceToHost));
@@ -491,7 +655,7 @@ int bpsx_random_points(bpsx_sim* sim, uint32_t scene, const float* u, uint32_t n
   char* b = (char*)sim->d_batch;
   float* d_in = (float*)b; float* d_xyz = (float*)(b + f3); uint32_t* d_ref = (uint32_t*)(b + 2 * f3);
   HIP_TRY(hipMemcpy(d_in, u, f3, hipMemcpyHostToDevice));
-  launch_random_points(sim->nav, scene, d_in, n, d_xyz, d_ref, nullptr);
+  launch_random_points(sim->nav, scene_entry(sim, scene), d_in, n, d_xyz, d_ref, nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipMemcpy(out_xyz, d_xyz, f3, hipMemcpyDeviceToHost));
   HIP_TRY(hipMemcpy(out_ref, d_ref, (size_t)n * 4, hipMemcpyDeviceToHost));

@@ -28,7 +28,13 @@ struct StepParams {
   float turn_left[4], turn_right[4];  // glm::angleAxis(+-radians(10), up), x,y,z,w
   uint32_t* error_flag;
   uint64_t* counters;
+  // scene rotation: per scene slot the scene-table entry its envs move to when their episode
+  // ends (kNoSwap: none) and how many envs have yet to move
+  uint32_t num_slots;
+  const uint32_t* swap_target;
+  uint32_t* swap_remaining;
 };
+constexpr uint32_t kNoSwap = 0xffffffffu;
 
 constexpr int kStepEvents = 5;  // timestamps recorded by launch_step when asked to
 

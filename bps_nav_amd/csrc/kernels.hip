@@ -232,7 +232,16 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
       }
       if (done) {
         // the terminal query above holds copies of the old episode's points: the pose arrays can
-        // take the next episode now; distance bookkeeping waits for step_finish
+        // take the next episode now; distance bookkeeping waits for step_finish.  If a new scene
+        // waits for this env's slot, the next episode is drawn there (simulator.cpp:1636-1642).
+        {
+          const uint32_t cur = A.scene[gi], tgt = P.swap_target[cur % P.num_slots];
+          if (tgt != kNoSwap && tgt != cur) {
+            A.scene[gi] = tgt;
+            A.last_cost[gi] = 0;
+            atomicSub(&P.swap_remaining[cur % P.num_slots], 1u);
+          }
+        }
         begin_reset(nav, A, P, gi);
         reset = true;
       }

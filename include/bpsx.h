@@ -72,6 +72,8 @@ typedef struct bpsx_config {
   int32_t gpu_id;             /* HIP device ordinal                                        */
   uint32_t max_steps;         /* 0 => BPSX_MAX_STEPS                                       */
   uint32_t task;              /* BPSX_TASK_*                                               */
+  float scene_reserve;        /* space for scene rotation: capacity of the navmesh arrays as
+                                 a multiple of the initial scenes' total size; 0 => 3      */
 } bpsx_config;
 
 /* Output tensors of one group, device pointers that stay valid and fixed for the
@@ -111,6 +113,21 @@ int bpsx_add_scene(bpsx_sim *sim, const void *navmesh_bytes, size_t navmesh_size
  * N/num_active_scenes (simulator.cpp:1205-1221) and allocates state. */
 int bpsx_finalize(bpsx_sim *sim);
 void bpsx_destroy(bpsx_sim *sim);
+
+/* Scene rotation (SceneSwapper / SceneTracker, simulator.cpp:1063-1178, 1284-1310, 1636-1642):
+ * swap_scene uploads a new scene for scene slot `slot` (0..num_active_scenes-1).  From then
+ * on every env of that slot moves to the new scene, with its episode table, when its episode
+ * ends (not on an explicit reset); the old scene stays resident meanwhile.  One swap per slot
+ * at a time: BPSX_E_STATE while envs are still on the old scene (the reference's
+ * canSwapScene()).  The reference loads in a background thread and picks the scene at random;
+ * here the caller chooses the scene and the call returns when it is resident.  Must not be
+ * called between step_start and step_end.  BPSX_E_UNSUPPORTED if the scene does not fit the
+ * space reserved at finalize (bpsx_config.scene_reserve). */
+int bpsx_swap_scene(bpsx_sim *sim, uint32_t slot, const void *navmesh_bytes, size_t navmesh_size,
+                    const float *episodes, uint32_t num_episodes);
+/* Envs of the slot that are still on the old scene (0: no swap in progress), and the number
+ * of swaps completed over all slots since creation (swap_stats, simulator.cpp:1412-1424). */
+int bpsx_swap_status(bpsx_sim *sim, uint32_t slot, uint32_t *envs_remaining, uint64_t *swaps_completed);
 
 /* ---- stepping (simulator.cpp:1377-1410) ---- */
 int bpsx_num_groups(const bpsx_sim *sim, uint32_t *out);

@@ -130,6 +130,12 @@ struct ApiImpl {
   }                                                                                                         \
   BPO_API void bpo_sim_set_task(void* h, uint32_t task) { ((ApiImpl<B>::SimT*)h)->setTask(task); }         \
   BPO_API int bpo_sim_finalize(void* h) { return ApiImpl<B>::sim_finalize(h); }                             \
+  BPO_API int bpo_sim_swap_scene(void* h, uint32_t slot, const void* b, size_t n, const float* ep, uint32_t E) { \
+    return ((ApiImpl<B>::SimT*)h)->swapScene(slot, (const uint8_t*)b, n, ep, E, &ApiImpl<B>::err()) ? 0 : -1; \
+  }                                                                                                         \
+  BPO_API uint32_t bpo_sim_swap_remaining(void* h, uint32_t slot) {                                        \
+    return ((ApiImpl<B>::SimT*)h)->swapRemaining(slot);                                                     \
+  }                                                                                                         \
   BPO_API uint32_t bpo_sim_envs_per_group(void* h) { return ((ApiImpl<B>::SimT*)h)->envsPerGroup(); }      \
   BPO_API void bpo_sim_reset(void* h, uint32_t g) { ((ApiImpl<B>::SimT*)h)->reset(g); }                    \
   BPO_API void bpo_sim_step(void* h, uint32_t g, const int64_t* a) { ((ApiImpl<B>::SimT*)h)->step(g, a); } \

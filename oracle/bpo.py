@@ -46,6 +46,9 @@ class Lib:
         L.bpo_sim_add_scene.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t, _f32p, C.c_uint32]
         L.bpo_sim_finalize.argtypes = [C.c_void_p]
         L.bpo_sim_set_task.argtypes = [C.c_void_p, C.c_uint32]
+        L.bpo_sim_swap_scene.argtypes = [C.c_void_p, C.c_uint32, C.c_char_p, C.c_size_t, _f32p, C.c_uint32]
+        L.bpo_sim_swap_remaining.argtypes = [C.c_void_p, C.c_uint32]
+        L.bpo_sim_swap_remaining.restype = C.c_uint32
         L.bpo_sim_envs_per_group.argtypes = [C.c_void_p]
         L.bpo_sim_envs_per_group.restype = C.c_uint32
         L.bpo_sim_reset.argtypes = [C.c_void_p, C.c_uint32]
@@ -172,6 +175,14 @@ class Sim:
 
     def __del__(self):
         self.close()
+
+    def swap_scene(self, slot, blob, eps):
+        eps = np.ascontiguousarray(eps, np.float32).reshape(-1, 10)
+        if self.lib.L.bpo_sim_swap_scene(self.h, slot, blob, len(blob), eps, len(eps)) != 0:
+            raise RuntimeError("swap_scene failed: " + self.lib.error())
+
+    def swap_remaining(self, slot):
+        return int(self.lib.L.bpo_sim_swap_remaining(self.h, slot))
 
     def reset(self, group=0):
         self.lib.L.bpo_sim_reset(self.h, group)

@@ -10,6 +10,9 @@
 //   computeGeoDist                                                   simulator.cpp:553-563
 //   RolloutGenerator::simulate / simulateStart / simulateEnd         simulator.cpp:1619-1700
 //   EnvironmentGroup env->scene assignment                           simulator.cpp:1205-1221
+//   scene rotation (SceneSwapper, SceneTracker, swapReady/swapScene)  simulator.cpp:1063-1178, 1284-1310, 1636-1642
+//     (the reference loads the next scene in a background thread and picks it at random; here
+//      the caller names it, like the engine's bpsx_swap_scene)
 // glm closed forms (angleAxis, quat*quat, quat*vec3, mat3_cast) are written out; glm is
 // not vendored by the reference, so those are "parity unpinned" and pinned here by closed
 // forms in tests/test_oracle_closed_forms.py.  The same holds for glm::inverse(quat) =
@@ -102,7 +105,8 @@ struct TurnConstants {
 };
 
 struct Env {
-  uint32_t scene = 0;
+  uint32_t scene = 0;   // index into the simulator's scene list
+  uint32_t slot = 0;    // scene slot the env belongs to (fixed)
   float pos[3] = {0, 0, 0}, rot[4] = {0, 0, 0, 1}, goal[3] = {0, 0, 0};
   NavPt nav{{0, 0, 0}, 0}, navGoal{{0, 0, 0}, 0};
   uint32_t step = 0;
@@ -142,6 +146,28 @@ class Sim {
         seed_(seed), maxSteps_(maxSteps ? maxSteps : 500), numThreads_(numThreads < 1 ? 1 : numThreads) {}
   ~Sim() { stopWorkers(); }
   void setTask(uint32_t task) { task_ = task; }
+  // Starts a swap of scene slot `slot`: its envs move to the new scene when their episode ends.
+  // False while the previous swap of the slot is in progress.
+  bool swapScene(uint32_t slot, const uint8_t* bytes, size_t n, const float* episodes, uint32_t numEpisodes,
+                 std::string* err) {
+    if (slot >= numScenes_) { *err = "slot out of range"; return false; }
+    if (swapRemaining_[slot]) { *err = "previous swap still in progress"; return false; }
+    auto sc = B::load(bytes, n, err);
+    if (!sc) return false;
+    scenes_.push_back(sc);
+    SceneEpisodes e;
+    e.count = numEpisodes;
+    e.rows.assign(episodes, episodes + (size_t)numEpisodes * 10);
+    episodes_.push_back(std::move(e));
+    swapTarget_[slot] = (uint32_t)scenes_.size() - 1;
+    swapRemaining_[slot] = numEnvs_ / numScenes_;
+    // the query contexts are per thread and per scene: rebuild them with the new scene
+    std::vector<std::thread> builders;
+    for (int t = 0; t < numThreads_; ++t) builders.emplace_back([this, t] { ctxs_[t] = B::make_ctx(scenes_); });
+    for (auto& b : builders) b.join();
+    return true;
+  }
+  uint32_t swapRemaining(uint32_t slot) const { return slot < numScenes_ ? swapRemaining_[slot].load() : 0; }
 
   bool addScene(const uint8_t* bytes, size_t n, const float* episodes, uint32_t numEpisodes, std::string* err) {
     auto s = B::load(bytes, n, err);
@@ -163,7 +189,10 @@ class Sim {
     // group g owns scenes [g*S/G, (g+1)*S/G) and, per scene, a contiguous block of N/S envs
     envs_.assign(numEnvs_, Env());
     const uint32_t envsPerScene = numEnvs_ / numScenes_;
-    for (uint32_t i = 0; i < numEnvs_; ++i) envs_[i].scene = i / envsPerScene;
+    for (uint32_t i = 0; i < numEnvs_; ++i) { envs_[i].scene = i / envsPerScene; envs_[i].slot = i / envsPerScene; }
+    swapTarget_.assign(numScenes_, 0xffffffffu);
+    swapRemaining_ = std::vector<std::atomic<uint32_t>>(numScenes_);
+    for (auto& r : swapRemaining_) r.store(0);
     rewards_.assign(numEnvs_, 0.f);
     masks_.assign(numEnvs_, 0);
     infos_.assign((size_t)numEnvs_ * 3, 0.f);
@@ -353,6 +382,12 @@ class Sim {
       if (curReset_) {
         resetEnv(gi, c);
       } else if (stepEnv(gi, curActions_[i], c)) {
+        Env& e = envs_[gi];
+        const uint32_t tgt = swapTarget_[e.slot];
+        if (tgt != 0xffffffffu && e.scene != tgt) {   // swapReady / swapScene
+          e.scene = tgt;
+          swapRemaining_[e.slot].fetch_sub(1);
+        }
         resetEnv(gi, c);
       }
     }
@@ -400,6 +435,8 @@ class Sim {
   }
 
   uint32_t task_ = TASK_POINTNAV;
+  std::vector<uint32_t> swapTarget_;
+  std::vector<std::atomic<uint32_t>> swapRemaining_;
   uint32_t numEnvs_, numScenes_, groups_, resetMode_;
   uint64_t seed_;
   uint32_t maxSteps_;

@@ -320,6 +320,53 @@ def test_full_size_workload_properties(oracle, torch_cuda):
     assert (d[fin] >= r["polar"][fin, 0] * 0.98 - 0.5).all(), "a path shorter than the straight line"
 
 
+def test_scene_rotation_parity(oracle, torch_cuda):
+    """Scenes are swapped in while the simulation runs (SceneSwapper, simulator.cpp:1063-1154):
+    envs move to the new scene when their episode ends.  Same swaps at the same steps on the
+    oracle; everything must stay equal, through several generations per slot, with scenes of
+    different sizes (the engine re-uses the space of scenes that left)."""
+    from oracle import bpo
+    print("case: scene rotation", flush=True)
+    pool = common.build_scenes(oracle, 2, 6, episodes_per_scene=24) + common.build_scenes(oracle, 1, 2, episodes_per_scene=24)
+    n, S = 96, 3
+    cpu = bpo.Sim(oracle, pool[:S], n, seed=5, threads=3, max_steps=40)
+    gen = make_gen(pool[:S], n, seed=5, max_steps=40, scene_reserve=4.0)
+    cpu.reset()
+    gen.reset(0)
+    state, infos = gen.get_state(0), gen.get_infos(0)
+    nxt = S
+    swaps = 0
+    for t, a in enumerate(common.action_stream(2, 420, n)):
+        if t % 25 == 10:
+            for slot in range(S):
+                rem, _ = gen.swap_status(slot)
+                assert rem == cpu.swap_remaining(slot)
+                if rem == 0:
+                    blob, eps = pool[nxt % len(pool)]
+                    nxt += 1
+                    cpu.swap_scene(slot, blob, eps)
+                    gen.swap_scene(slot, blob, eps)
+                    swaps += 1
+                else:
+                    with pytest.raises(RuntimeError, match="still in progress"):
+                        gen.swap_scene(slot, *pool[0])
+        cpu.step(a)
+        gen.step(0, a)
+        co, cs = cpu.outputs(), cpu.state()
+        st = {k: v.cpu().numpy() for k, v in state.items()}
+        for k in ("poly_ref", "goal_ref", "step", "episode", "num_resets"):
+            assert np.array_equal(cs[k], st[k].view(np.uint32)), f"{k} differs at step {t}"
+        assert np.array_equal(common.bits(st["position"]), common.bits(cs["position"])), f"position at step {t}"
+        assert np.array_equal(co["masks"], gen.get_masks(0).cpu().numpy())
+        gi = infos.packed.cpu().numpy()
+        assert np.array_equal(common.bits(gi), common.bits(co["infos"])) or np.isnan(gi).any(), f"infos at step {t}"
+    assert swaps >= 12
+    assert gen.swap_status(0)[1] >= 6, "swaps did not complete"
+    assert gen.swap_stats[0] > 0
+    gen.check_errors()
+    gen.close()
+
+
 def test_error_paths(oracle, torch_cuda):
     print("case: error paths", flush=True)
     sc = common.build_scenes(oracle, 1, 1, episodes_per_scene=8)

@@ -341,6 +341,34 @@ def test_exploration_reward_is_quarter_per_new_cell(oracle):
     assert total == pytest.approx(0.25 * sim.outputs()["infos"][0, 0]) and sim.outputs()["infos"][0, 0] == 3.0
 
 
+def test_scene_rotation_moves_envs_when_their_episode_ends(oracle):
+    # SceneSwapper / swapReady / swapScene (simulator.cpp:1063-1154, 1284-1310, 1636-1642): after a
+    # swap is started, an env changes scene exactly when its episode ends; an explicit reset does not.
+    room = meshes.l_shape()
+    other = meshes.two_rooms()
+    ep_room = np.concatenate([(2, 0, 2), episodes.yaw_quat(np.array(0.0)), (2, 0, 8)]).astype(np.float32)[None]
+    ep_other = np.concatenate([(1, 0, 1), episodes.yaw_quat(np.array(0.0)), (1, 0, 2)]).astype(np.float32)[None]
+    sim = bpo.Sim(oracle, [(room, ep_room)], 4, max_steps=6)
+    sim.reset()
+    sim.swap_scene(0, other, ep_other)
+    assert sim.swap_remaining(0) == 4
+    with pytest.raises(RuntimeError, match="in progress"):
+        sim.swap_scene(0, other, ep_other)
+    sim.reset()                                   # not an episode end: nobody moves
+    assert sim.swap_remaining(0) == 4
+    assert np.allclose(sim.state()["position"], (2, 0, 2), atol=1e-5)
+    sim.step(np.array([2, 0, 2, 2]))              # env 1 stops: it alone moves to the new scene
+    assert sim.swap_remaining(0) == 3
+    pos = sim.state()["position"]
+    assert np.allclose(pos[1], (1, 0, 1), atol=1e-5) and np.allclose(pos[[0, 2, 3]], (2, 0, 2), atol=1e-5)
+    for _ in range(5):                            # the others run into max_steps
+        sim.step(np.array([2, 2, 2, 2]))
+    assert sim.swap_remaining(0) == 0
+    assert np.allclose(sim.state()["position"], (1, 0, 1), atol=1e-5)
+    sim.swap_scene(0, room, ep_room)              # and back again: allowed now
+    assert sim.swap_remaining(0) == 4
+
+
 def test_invalid_action_is_flagged_and_agent_untouched(oracle):
     sim = one_room_sim(oracle)
     sim.reset()
