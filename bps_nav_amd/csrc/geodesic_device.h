@@ -158,8 +158,11 @@ struct GeoWave {
     wave_sync();
   }
   // node index of polygon ip, or -1 (any lane, independently); one LDS access per chain step
-  template <bool S> BPSX_DEV int find(uint32_t ip, uint32_t bucket) const {
-    for (uint32_t i = L->first[bucket]; i != kChainEnd;) {
+  // *head receives the bucket's first node (what a new node of this bucket links to)
+  template <bool S> BPSX_DEV int find(uint32_t ip, uint32_t bucket, uint32_t* head) const {
+    const uint32_t h = L->first[bucket];
+    *head = h;
+    for (uint32_t i = h; i != kChainEnd;) {
       const uint32_t l = link<S>((int)i);
       if (link_id(l) == ip) return (int)i;
       i = link_next(l);
@@ -423,7 +426,8 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
     int ni = -1;
-    if (nb != kNoNb) ni = g.find<S>(nb, bucket);
+    uint32_t chainHead = kChainEnd;
+    if (nb != kNoNb) ni = g.find<S>(nb, bucket, &chainHead);
     // the polygon the expanded node was reached from is not entered again
     if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
     PHASE_MARK(3);
@@ -443,10 +447,9 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       // hash insertion by all new nodes at once; of two that share a bucket one store wins
       // and the other lane goes round again behind it
       bool pending = isNew && nb != kNoNb;
-      if ((need & (need - 1)) == 0) {   // one new node: no other lane can take its bucket
+      if ((need & (need - 1)) == 0) {   // one new node: the chain head seen by its lookup still stands
         if (pending) {
-          const uint32_t head = L->first[bucket];
-          g.set_link<S>(ni, nb | (head << 16));
+          g.set_link<S>(ni, nb | (chainHead << 16));
           L->first[bucket] = (uint16_t)ni;
         }
         pending = false;
