@@ -14,12 +14,14 @@
 //     older node is simply read from there.
 // Heap entries beyond kHeapLds and links beyond kLinksLds spill to the same slot.  A query
 // runs the instantiation of the loop without spill code until one more expansion could
-// outgrow the links in LDS or the register heap, then carries on in a spilling instantiation.  Per expanded node the
-// regular HBM traffic is the polygon's six 16-byte edge records (lane j of the wavefront
-// handles edge j: node lookup, cost, heuristic) plus the write-through of updated nodes; heap
-// updates are applied in edge order, which is what makes the result identical to the
-// sequential algorithm, ties included.  Everything that is the same for all lanes (heap walks,
-// counters, the expanded node) is kept in scalar registers and branches on the scalar unit.
+// outgrow the links in LDS or the register heap, then carries on in a spilling instantiation.
+// Per expanded node the regular HBM traffic is the polygon's six 16-byte edge records (lane j
+// of the wavefront handles edge j: node lookup, cost, heuristic) plus the write-through of
+// updated nodes; heap updates are applied in edge order, which is what makes the result
+// identical to the sequential algorithm, ties included.  A wavefront spends its time in one
+// chain of dependent steps, so the code is written for few of them: heap pops and pushes are
+// done by all lanes at once, what is the same for all lanes lives in scalar registers, and
+// LDS and HBM accesses stay separate instructions.
 //
 // Reference semantics followed: DetourNavMeshQuery.cpp:945-1178 (findPath, getPathToNode),
 // :1661-1696, 1765-1994 (appendVertex, findStraightPath), :2279-2381 (getPortalPoints,
@@ -170,7 +172,8 @@ struct GeoWave {
     return -1;
   }
 
-  // ---------------------------------------------------------------- open list
+  // ---------------------------------------------------------------- open list, once it has
+  // left the registers (more than kRegHeap entries: rare)
   // The heap is walked with wave-uniform indices: every lane issues the same LDS access and the
   // values are moved to scalar registers, so the loops below branch on the scalar unit and cost
   // a handful of vector instructions per level.
@@ -245,9 +248,9 @@ struct GeoWave {
 
 // The open list in registers.  Heap position q (1-based, root = 1; the reference's index + 1)
 // lives in lane q & 63 of the first register pair (q < 64) or of the second (64 <= q < 128).
-// Totals are kept as bit patterns and compared as unsigned integers on the scalar unit: they
-// are sums of distances, never negative and never NaN, and for such floats the integer order
-// of the bits is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
+// Totals are kept as bit patterns and compared as unsigned integers: they are sums of
+// distances, never negative and never NaN, and for such floats the integer order of the bits
+// is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
 constexpr int kRegHeap = 127;
 static_assert(kMaxNodes <= 2048, "heap entries keep the node index in 11 bits");
 static_assert(kHeapLds > kRegHeap, "the register heap must fit the LDS heap it is moved to");
