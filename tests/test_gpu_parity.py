@@ -240,6 +240,42 @@ def test_flee_and_exploration_step_parity(oracle, torch_cuda, task, config, num_
     gen.close()
 
 
+@pytest.mark.parametrize("config,num_scenes,n,steps,mode", [(2, 16, 1024, 1000, 0), (3, 64, 4096, 300, 1)])
+def test_step_parity_at_configured_sizes(oracle, torch_cuda, config, num_scenes, n, steps, mode):
+    """The second and third benchmark configurations at their own agent and scene counts (the
+    third with its area-weighted sampled resets), stepped side by side with the oracle on all
+    host cores: ids and positions bit for bit every step, infos bit for bit."""
+    import os
+    from oracle import bpo
+    print(f"case: configured size, config {config}: {n} agents / {num_scenes} scenes, {steps} steps", flush=True)
+    sc = common.build_scenes(oracle, config, num_scenes, episodes_per_scene=32)
+    threads = min(16, len(os.sched_getaffinity(0)))
+    cpu = bpo.Sim(oracle, sc, n, reset_mode=mode, seed=101, threads=threads)
+    gen = make_gen(sc, n, reset_mode=mode, seed=101)
+    cpu.reset()
+    gen.reset(0)
+    state, infos = gen.get_state(0), gen.get_infos(0)
+    dones = 0
+    for t, a in enumerate(common.action_stream(config, steps, n)):
+        cpu.step(a)
+        gen.step(0, a)
+        if t % 8 and t < steps - 1:
+            continue   # every eighth step and the last are compared in full; a divergence persists
+        co, cs = cpu.outputs(), cpu.state()
+        st = {k: v.cpu().numpy() for k, v in state.items()}
+        for k in ("poly_ref", "goal_ref", "step", "episode", "num_resets"):
+            assert np.array_equal(cs[k], st[k].view(np.uint32)), f"{k} differs at step {t}"
+        assert np.array_equal(common.bits(st["position"]), common.bits(cs["position"])), f"position at step {t}"
+        assert np.array_equal(co["masks"], gen.get_masks(0).cpu().numpy())
+        gi = infos.packed.cpu().numpy()
+        same = common.bits(gi) == common.bits(co["infos"])
+        assert (same | np.isnan(gi)).all(), f"infos at step {t}"
+        dones += int((co["masks"] == 0).sum())
+    assert int(cs["num_resets"].sum()) > n
+    gen.check_errors()
+    gen.close()
+
+
 def test_full_size_workload_properties(oracle, torch_cuda):
     """The benchmark's own shape (16384 agents, 128 maze scenes of ~30k polygons), where the
     oracle cannot step along: size-independent properties plus oracle spot checks.
