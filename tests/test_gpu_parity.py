@@ -276,6 +276,65 @@ def test_step_parity_at_configured_sizes(oracle, torch_cuda, config, num_scenes,
     gen.close()
 
 
+def test_mixed_scenes_at_the_largest_configured_shape(oracle, torch_cuda):
+    """The fifth benchmark configuration's shape: 65536 agents over 256 scenes of mixed kinds and
+    sizes in one simulator (room plans, cluttered plans, mazes of ~30k polygons, and the
+    Recast-built two-floor mesh with its ramp), stepped next to the oracle.  Scenes stay within
+    what one Detour tile holds (32767 polygons), which is all the reference's PathFinder supports."""
+    import os
+    from bps_nav_amd import episodes, scenes
+    from bps_nav_amd.bps_sim import nav_only
+    from oracle import bpo
+    print("case: 65536 agents / 256 mixed scenes", flush=True)
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    with open(os.path.join(gold, "recast_two_floors.navmesh"), "rb") as f:
+        two_floors = f.read()
+    blobs, ranges = [], []
+    for i in range(256):
+        kind = i % 8
+        if kind < 3:
+            blobs.append(scenes.config_scene(2, i)); ranges.append((1.0, 30.0))
+        elif kind < 6:
+            blobs.append(scenes.config_scene(3, i)); ranges.append((1.0, 30.0))
+        elif kind == 6:
+            blobs.append(scenes.config_scene(4, i)); ranges.append((5.0, 30.0))
+        else:
+            blobs.append(two_floors); ranges.append((1.0, 30.0))
+    nav = nav_only(blobs)
+
+    def gfn(i):
+        def f(s, g):
+            sx, sr = nav.snap_points(i, s)
+            gx, gr = nav.snap_points(i, g)
+            return nav.geodesic(i, sx, sr, gx, gr)
+        return f
+    sc = [(b, episodes.make_episodes(b, 2000 + i, 32, ranges[i][0], ranges[i][1], gfn(i))) for i, b in enumerate(blobs)]
+    nav.close()
+    n, steps = 65536, 60
+    threads = min(16, len(os.sched_getaffinity(0)))
+    cpu = bpo.Sim(oracle, sc, n, seed=55, threads=threads)
+    gen = make_gen(sc, n, seed=55)
+    cpu.reset()
+    gen.reset(0)
+    rng = np.random.default_rng(8)
+    for t in range(steps):
+        a = episodes.random_actions(rng, n, 0.7)
+        cpu.step(a)
+        gen.step(0, a)
+    co, cs = cpu.outputs(), cpu.state()
+    st = {k: v.cpu().numpy() for k, v in gen.get_state(0).items()}
+    for k in ("poly_ref", "goal_ref", "step", "episode", "num_resets"):
+        assert np.array_equal(cs[k], st[k].view(np.uint32)), f"{k} differs"
+    assert np.array_equal(common.bits(st["position"]), common.bits(cs["position"]))
+    gi = gen.get_infos(0).packed.cpu().numpy()
+    assert ((common.bits(gi) == common.bits(co["infos"])) | np.isnan(gi)).all()
+    assert np.array_equal(co["masks"], gen.get_masks(0).cpu().numpy())
+    assert int(cs["num_resets"].sum()) > n
+    assert (st["position"][:, 1] > 2.0).any(), "nobody on the upper floor of the two-floor scenes"
+    gen.check_errors()
+    gen.close()
+
+
 def test_full_size_workload_properties(oracle, torch_cuda):
     """The benchmark's own shape (16384 agents, 128 maze scenes of ~30k polygons), where the
     oracle cannot step along: size-independent properties plus oracle spot checks.
