@@ -473,53 +473,46 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
 #ifdef BPSX_QUERY_TRACE
     g.missNb += (uint32_t)__popcll(__ballot(nb != kNoNb && !isNew && !g.in_window(ni)));
 #endif
-    bool update = false, wasOpen = false;
-    float total = 0, heuristic = 0;
-    if (nb != kNoNb) {
-      float p0 = m0, p1 = m1, p2 = m2, oldTotal = 0;
-      uint32_t fl = 0;
-      const bool inw = g.in_window(ni);   // new nodes always are
-
-      const int w = ni & (kWindow - 1);
-      ANode& hn = g.ws->nodes[ni];
-      if (!isNew) {
-        fl = state_flags(g.state<S>(ni));
-        if (inw) {
-          p0 = L->w_pos[0][w]; p1 = L->w_pos[1][w]; p2 = L->w_pos[2][w]; oldTotal = L->w_total[w];
-        } else {
-          BPSX_KEEP_APART();
-          const float4 pc = *reinterpret_cast<const float4*>(hn.pos);   // pos, cost
-          const float2 ts = *reinterpret_cast<const float2*>(&hn.total);  // total, state
-          p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = ts.x;
-          BPSX_KEEP_APART();
-        }
+    // Costs of the step to each neighbour (lane-wise).  Written with few branches: all lanes
+    // issue the one round of LDS reads a revisited node needs (idle lanes read slot 0), the rare
+    // node that has left the window is fetched under a wave-uniform test, new nodes take the
+    // portal midpoint instead, and everything is stored in one predicated block.
+    const bool valid = nb != kNoNb;
+    const int nis = valid ? ni : 0;
+    const int w = nis & (kWindow - 1);
+    const bool inw = g.in_window(nis);   // new nodes always are
+    ANode& hn = g.ws->nodes[nis];
+    uint32_t fl = state_flags(g.state<S>(nis));
+    float p0 = L->w_pos[0][w], p1 = L->w_pos[1][w], p2 = L->w_pos[2][w], oldTotal = L->w_total[w];
+    const bool miss = valid && !isNew && !inw;
+    if (__ballot(miss)) {
+      if (miss) {
+        BPSX_KEEP_APART();
+        const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
+        const float2 ts = *reinterpret_cast<const float2*>(&hn.total);  // total, state
+        p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = ts.x;
+        BPSX_KEEP_APART();
       }
-      const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
-      const float curCost = sqrtf(cx * cx + cy * cy + cz * cz) * 1.0f;
-      const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
-      const float toEnd = sqrtf(ex * ex + ey * ey + ez * ez);
-      float cost;
-      if (nb == endIp) {
-        cost = bcost + curCost + toEnd * 1.0f;
-        heuristic = 0;
-      } else {
-        cost = bcost + curCost;
-        heuristic = toEnd * H_SCALE;
+    }
+    if (isNew) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }
+    const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
+    const float curCost = sqrtf(cx * cx + cy * cy + cz * cz) * 1.0f;
+    const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
+    const float toEnd = sqrtf(ex * ex + ey * ey + ez * ez);
+    const bool last = nb == endIp;
+    const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
+    const float heuristic = last ? 0.0f : toEnd * H_SCALE;
+    const float total = cost + heuristic;
+    const bool update = valid && !(fl && total >= oldTotal);
+    const bool wasOpen = update && (fl & 1u) != 0;
+    if (update) {
+      g.set_state<S>(ni, 1u | ((uint32_t)(bi + 1) << 2));   // open, parent = expanded node
+      if (inw) {
+        L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2;   // unchanged for a revisited node
+        L->w_cost[w] = cost; L->w_total[w] = total;
       }
-      total = cost + heuristic;
-      const bool worse = fl && total >= oldTotal;
-      if (!worse) {
-        update = true;
-        wasOpen = (fl & 1u) != 0;
-        g.set_state<S>(ni, 1u | ((uint32_t)(bi + 1) << 2));   // open, parent = expanded node
-        if (inw) {
-          if (isNew) { L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2; }
-          L->w_cost[w] = cost; L->w_total[w] = total;
-        }
-        if (isNew) *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
-        else hn.cost = cost;
-        hn.total = total;
-      }
+      *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
+      hn.total = total;
     }
     wave_sync();
     PHASE_MARK(5);
