@@ -160,16 +160,22 @@ struct GeoWave {
     wave_sync();
   }
   // node index of polygon ip, or -1 (any lane, independently); one LDS access per chain step
-  // *head receives the bucket's first node (what a new node of this bucket links to)
-  template <bool S> BPSX_DEV int find(uint32_t ip, uint32_t bucket, uint32_t* head) const {
-    const uint32_t h = L->first[bucket];
-    *head = h;
-    for (uint32_t i = h; i != kChainEnd;) {
-      const uint32_t l = link<S>((int)i);
-      if (link_id(l) == ip) return (int)i;
-      i = link_next(l);
+  // Node index of polygon ip, or -1; *head receives the bucket's first node (what a new node of
+  // this bucket links to).  Called by all lanes (idle ones with valid = false): the chains are
+  // walked in step, one LDS access per lane and round, until every lane has hit or run out.
+  template <bool S> BPSX_DEV int find(bool valid, uint32_t ip, uint32_t bucket, uint32_t* head) const {
+    uint32_t cur = L->first[bucket];
+    if (!valid) cur = kChainEnd;
+    *head = cur;
+    int found = -1;
+    while (__ballot(cur != kChainEnd)) {
+      const bool live = cur != kChainEnd;
+      const uint32_t l = link<S>(live ? (int)cur : 0);
+      const bool hit = live && link_id(l) == ip;
+      found = hit ? (int)cur : found;
+      cur = (live && !hit) ? link_next(l) : kChainEnd;
     }
-    return -1;
+    return found;
   }
 
   // ---------------------------------------------------------------- open list, once it has
@@ -428,9 +434,8 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
-    int ni = -1;
-    uint32_t chainHead = kChainEnd;
-    if (nb != kNoNb) ni = g.find<S>(nb, bucket, &chainHead);
+    uint32_t chainHead;
+    int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead);
     // the polygon the expanded node was reached from is not entered again
     if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
     PHASE_MARK(3);
