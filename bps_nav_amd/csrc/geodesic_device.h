@@ -440,39 +440,41 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
     PHASE_MARK(3);
     // new nodes take consecutive indices in edge order; past the pool's end they are dropped
-    const unsigned long long need = __ballot(nb != kNoNb && ni < 0);
-    const bool isNew = (need >> lane) & 1ull;
+    const bool isNew = nb != kNoNb && ni < 0;
+    const unsigned long long need = __ballot(isNew);
     if (need) {
-      const int rank = __popcll(need & ((1ull << lane) - 1ull));
+      const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
+      const int count = __popcll(need);
       if (isNew) {
         const int idx = g.nodeCount + rank;
         if (!S || idx < kMaxNodes) ni = idx;
         else nb = kNoNb;
       }
-      const int want = g.nodeCount + __popcll(need);
+      const int want = g.nodeCount + count;
       if (S && want > kMaxNodes) st.outOfNodes = true;
       g.nodeCount = (!S || want < kMaxNodes) ? want : kMaxNodes;
-      // hash insertion by all new nodes at once; of two that share a bucket one store wins
-      // and the other lane goes round again behind it
       bool pending = isNew && nb != kNoNb;
-      if ((need & (need - 1)) == 0) {   // one new node: the chain head seen by its lookup still stands
+      if (count == 1) {
+        // one new node: the chain head seen by its lookup still stands
         if (pending) {
           g.set_link<S>(ni, nb | (chainHead << 16));
           L->first[bucket] = (uint16_t)ni;
         }
-        pending = false;
-        wave_sync();
-      }
-      while (__ballot(pending)) {
-        if (pending) {
-          const uint32_t head = L->first[bucket];
-          g.set_link<S>(ni, nb | (head << 16));
-          L->first[bucket] = (uint16_t)ni;
+      } else {
+        // several: all insert at once; of two that share a bucket one store wins and the other
+        // lane goes round again behind it
+        while (__ballot(pending)) {
+          if (pending) {
+            const uint32_t head = L->first[bucket];
+            g.set_link<S>(ni, nb | (head << 16));
+            L->first[bucket] = (uint16_t)ni;
+          }
+          wave_sync();
+          if (pending && L->first[bucket] == (uint16_t)ni) pending = false;
+          wave_sync();
         }
-        wave_sync();
-        if (pending && L->first[bucket] == (uint16_t)ni) pending = false;
-        wave_sync();
       }
+      wave_sync();
     }
     PHASE_MARK(4);
 #ifdef BPSX_QUERY_TRACE
