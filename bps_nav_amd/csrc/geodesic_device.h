@@ -322,19 +322,19 @@ struct RegHeap {
     const bool wide = size >= 64;           // entries in the second pair
     const bool lo = lane < 32;              // children of positions 32..63 are in the second pair
     const int c0 = (2 * lane) & 63;
+    // keys and nodes of both children in one round of cross-lane reads
     uint32_t cl = xlane(c0, t0), cr = xlane(c0 + 1, t0);
-    uint32_t hl = kEmpty, hr = kEmpty;
-    if (wide) { hl = xlane(c0, t1); hr = xlane(c0 + 1, t1); }
-    cl = lo ? cl : hl;
-    cr = lo ? cr : hr;
+    uint32_t nl = xlane(c0, n0), nr = xlane(c0 + 1, n0);
+    if (wide) {
+      const uint32_t hl = xlane(c0, t1), hr = xlane(c0 + 1, t1), ml = xlane(c0, n1), mr = xlane(c0 + 1, n1);
+      cl = lo ? cl : hl; cr = lo ? cr : hr; nl = lo ? nl : ml; nr = lo ? nr : mr;
+    } else {
+      cl = lo ? cl : kEmpty; cr = lo ? cr : kEmpty;
+    }
     const bool right = cr < cl;
     const uint32_t cmin = right ? cr : cl;
+    const uint32_t cn = right ? nr : nl;
     const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);   // position 2..127
-    uint32_t cn = xlane((int)(choice & 63), n0);
-    if (wide) {
-      const uint32_t hn = xlane((int)(choice & 63), n1);
-      cn = lo ? cn : hn;
-    }
     // route of the hole: 1, choice[1], choice[choice[1]], ...
     unsigned long long route = 2ull;
     uint32_t q = 1;
@@ -523,26 +523,33 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     wave_sync();
     PHASE_MARK(5);
-    // ---- ordered phase: heap and "nearest so far" updates in edge order
-    unsigned long long upd = __ballot(update);
-    const unsigned long long openMask = __ballot(update && wasOpen);
+    // ---- ordered phase, in edge order.  First the "nearest so far" record (lastBestNode of
+    // findPath): an update replaces it when its heuristic is lower; only lanes below the
+    // current record can matter, usually none.
     const uint32_t packed = (uint32_t)ni | (nb << 11);   // heap entry of this lane's node
+    unsigned long long better = __ballot(update && heuristic < st.lastBestCost);
+    while (better) {
+      const int src = __ffsll((long long)better) - 1;
+      better &= better - 1;
+      const float h = lane_f(heuristic, src);
+      if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
+    }
+    // then the open list
+    unsigned long long upd = __ballot(update);
+    const unsigned long long openMask = __ballot(wasOpen);
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
       const uint32_t entry = rlane(packed, src);
-      const int node = (int)(entry & 0x7ffu);
       const float t = lane_f(total, src);
-      const float h = lane_f(heuristic, src);
       const bool open = (openMask >> src) & 1ull;
       if (SH) {
-        if (open) g.modify<true>(node, t);
-        else g.push<true>(t, node);
+        if (open) g.modify<true>((int)(entry & 0x7ffu), t);
+        else g.push<true>(t, (int)(entry & 0x7ffu));
       } else {
         if (open) rh.modify(entry, __float_as_uint(t), lane);
         else rh.push(__float_as_uint(t), entry, lane);
       }
-      if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = node; }
     }
     PHASE_MARK(6);
   }
