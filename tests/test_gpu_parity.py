@@ -484,6 +484,22 @@ def test_error_paths(oracle, torch_cuda):
         gen.check_errors()
     with pytest.raises(RuntimeError):
         gen.rgba(0)
+    # scene rotation: bad slot, bad mesh, call while a step is in flight, scene that does not fit
+    with pytest.raises(RuntimeError, match="slot out of range"):
+        gen.swap_scene(3, *sc[0])
+    with pytest.raises(RuntimeError, match="magic"):
+        gen.swap_scene(0, b"XXXX" + sc[0][0][4:], sc[0][1])
+    gen.step_start(0, a)
+    with pytest.raises(RuntimeError, match="in flight"):
+        gen.swap_scene(0, *sc[0])
+    gen.step_end(0)
+    assert gen.swap_status(0) == (0, 0)
+    from bps_nav_amd import scenes as _sc
+    big = _sc.config_scene(3, 0)   # ~20k polygons against a reserve sized for a ~1.6k polygon room
+    with pytest.raises(RuntimeError, match="does not fit"):
+        gen.swap_scene(0, big, sc[0][1])
+    gen.swap_scene(0, *sc[0])       # a scene of the same size does
+    assert gen.swap_status(0)[0] == 8
     gen.close()
     from bps_nav_amd import scenes
     four = scenes.gen_scene(scenes.BOX_ROOM, 5, 5, size_x=10.0, size_z=10.0, num_boxes=4, box_min=0.5, box_max=2.0,
