@@ -51,7 +51,10 @@ namespace bpsx {
 constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link and state words are kept in LDS
 constexpr int kHeapLds = BPSX_HEAP_LDS;     // open-list entries kept in LDS
 constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
-constexpr int kHashSize = 512;
+#ifndef BPSX_HASH
+#define BPSX_HASH 512
+#endif
+constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash table
 static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
 
 BPSX_DEV void wave_sync() {
@@ -420,10 +423,11 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
 #ifdef BPSX_QUERY_TRACE
     if (!SH && (uint32_t)rh.size > g.maxHeap) g.maxHeap = (uint32_t)rh.size;
 #endif
-    const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)g.state<S>(bi)));
+    const uint32_t bstate = g.state<S>(bi);   // read now, moved to a scalar register only after the pop
     PHASE_MARK(0);
     if (SH) g.pop<true>();
     else rh.pop(lane);
+    const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)bstate));
     PHASE_MARK(1);
     g.set_state<S>(bi, 2u | (pidx << 2));   // open -> closed
     if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
