@@ -86,6 +86,31 @@ BPSX_DEV uint32_t wlane(uint32_t old, uint32_t v, int lane) {
   return old;
 }
 
+// lanes 8..15 of each row of 16 take src of the lane 8 below them, lanes 0..7 keep low
+BPSX_DEV float lanes_up8(float low, float src) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(low), __float_as_int(src), 0x118 /* row_shr:8 */, 0xf, 0xf, false));
+}
+// lanes 0..7 of each row take v of the lane 8 above them
+BPSX_DEV float lanes_down8(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x108 /* row_shl:8 */, 0xf, 0xf, false));
+}
+// Correctly rounded square root, the value sqrtf returns on the host: the hardware estimate is
+// within one unit in the last place, and the residuals of its two neighbours say which of the
+// three is the rounded root.  Same scheme as the compiler's own expansion of sqrtf, minus its
+// rescaling of arguments below 2^-96 (needed there for the residuals not to underflow): the
+// arguments here are squared distances, zero or far above that; a wavefront that meets one in
+// between takes the library routine.
+BPSX_DEV float sqrt_exact(float x) {
+  const uint32_t xb = __float_as_uint(x);
+  if (__ballot(xb - 1u < 0x0f800000u - 1u)) return sqrtf(x);   // 0 < x < 2^-96 in some lane: never in practice
+  const float s = __builtin_amdgcn_sqrtf(x);
+  const float down = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
+  const float rdown = fmaf(-down, s, x), rup = fmaf(-up, s, x);
+  float r = rdown <= 0.0f ? down : s;
+  r = rup > 0.0f ? up : r;
+  return r;
+}
+
 // LDS of one wavefront.
 struct GeoLds {
   uint16_t first[kHashSize];
@@ -302,9 +327,10 @@ struct RegHeap {
   // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
     const unsigned long long m0 = __ballot(lane >= 1 && lane <= size && n0 == n);
-    if (m0) { bubble_up(__ffsll((long long)m0) - 1, t, n, lane); return; }
-    const unsigned long long m1 = __ballot(64 + lane <= size && n1 == n);
-    if (m1) bubble_up(64 + __ffsll((long long)m1) - 1, t, n, lane);
+    const unsigned long long m1 = m0 ? 0ull : __ballot(64 + lane <= size && n1 == n);
+    if (!(m0 | m1)) return;
+    const int q = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
+    bubble_up(q, t, n, lane);
   }
   // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
   // by the root down to a leaf along the smaller children and then bubbles the former last
@@ -458,27 +484,24 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       if (S && want > kMaxNodes) st.outOfNodes = true;
       g.nodeCount = (!S || want < kMaxNodes) ? want : kMaxNodes;
       bool pending = isNew && nb != kNoNb;
-      if (count == 1) {
-        // one new node: the chain head seen by its lookup still stands
+      // All insert at once in front of the chain head their lookup saw.  Of several that share a
+      // bucket one store wins; the others see that when they read the head back and go round
+      // again behind the winner.  One new node needs no check.
+      uint32_t head = chainHead;
+      for (;;) {
         if (pending) {
-          g.set_link<S>(ni, nb | (chainHead << 16));
+          g.set_link<S>(ni, nb | (head << 16));
           L->first[bucket] = (uint16_t)ni;
         }
-      } else {
-        // several: all insert at once; of two that share a bucket one store wins and the other
-        // lane goes round again behind it
-        while (__ballot(pending)) {
-          if (pending) {
-            const uint32_t head = L->first[bucket];
-            g.set_link<S>(ni, nb | (head << 16));
-            L->first[bucket] = (uint16_t)ni;
-          }
-          wave_sync();
-          if (pending && L->first[bucket] == (uint16_t)ni) pending = false;
-          wave_sync();
+        wave_sync();
+        if (count == 1) break;
+        if (pending) {
+          head = L->first[bucket];
+          pending = head != (uint32_t)ni;
         }
+        wave_sync();
+        if (!__ballot(pending)) break;
       }
-      wave_sync();
     }
     PHASE_MARK(4);
 #ifdef BPSX_QUERY_TRACE
@@ -506,10 +529,13 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       }
     }
     if (isNew) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }
+    // both square roots in one pass: lanes 8..13 take the second operand of lanes 0..5
     const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
-    const float curCost = sqrtf(cx * cx + cy * cy + cz * cz) * 1.0f;
     const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
-    const float toEnd = sqrtf(ex * ex + ey * ey + ez * ez);
+    const float cc = cx * cx + cy * cy + cz * cz, ee = ex * ex + ey * ey + ez * ez;
+    const float roots = sqrt_exact(lanes_up8(cc, ee));
+    const float curCost = roots * 1.0f;
+    const float toEnd = lanes_down8(roots);
     const bool last = nb == endIp;
     const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
     const float heuristic = last ? 0.0f : toEnd * H_SCALE;
