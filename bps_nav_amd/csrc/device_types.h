@@ -169,6 +169,10 @@ constexpr __host__ __device__ uint32_t geo_class(uint32_t last_cost) {
                                                              : (uint32_t)kGeoClasses - 1u - last_cost / kGeoClassWidth;
 }
 constexpr uint32_t kGeoClassUnknown = geo_class(700);   // a search without history: upper-middle length
+// AgentArrays::last_cost before the episode's first goal -> agent search.  The distance taken at
+// reset is searched the other way round and the previous episode's searches had another goal:
+// neither says how long the first search will be, and it is often among the longest.
+constexpr uint32_t kCostUnknown = 0xffffffffu;
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,

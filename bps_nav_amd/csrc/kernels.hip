@@ -122,6 +122,7 @@ BPSX_DEV void begin_reset(const NavData& nav, const AgentArrays& A, const StepPa
   const uint32_t count = A.nresets[gi];
   A.nresets[gi] = count + 1;
   A.step[gi] = 1;
+  A.last_cost[gi] = kCostUnknown;
   const uint32_t sc = A.scene[gi];
   const SceneDev& s = nav.scenes[sc];
   const uint64_t key = reset_key(P.seed, gi, count);
@@ -225,10 +226,8 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
         q.out = gi;
         q.cost_slot = done ? kNoCostSlot : gi;   // a finished episode's search predicts nothing
         q.pad = 0;
-        cls = geo_class(A.last_cost[gi]);
-        // the first search of an episode ran the other way (agent -> goal) and says little about
-        // the cost of goal -> agent: assume an upper-middle length for the first step
-        if (step <= 2 && cls > kGeoClassUnknown) cls = kGeoClassUnknown;
+        const uint32_t expected = A.last_cost[gi];
+        cls = expected == kCostUnknown ? kGeoClassUnknown : geo_class(expected);
       }
       if (done) {
         // the terminal query above holds copies of the old episode's points: the pose arrays can
@@ -238,7 +237,6 @@ __global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, S
           const uint32_t cur = A.scene[gi], tgt = P.swap_target[cur % P.num_slots];
           if (tgt != kNoSwap && tgt != cur) {
             A.scene[gi] = tgt;
-            A.last_cost[gi] = 0;
             atomicSub(&P.swap_remaining[cur % P.num_slots], 1u);
           }
         }
@@ -404,7 +402,7 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
       q.b[0] = b.x; q.b[1] = b.y; q.b[2] = b.z; q.b_ref = b.ref;
       q.scene = A.scene[gi];
       q.out = P.total + gi;
-      q.cost_slot = gi;
+      q.cost_slot = kNoCostSlot;   // searched agent -> goal: says little about the searches to come
       q.pad = 0;
       // a new episode: no history
       Q.queries[(size_t)kGeoClassUnknown * Q.stride + atomicAdd(&Q.counts[kQGeo + kGeoClassUnknown], 1u)] = q;
@@ -472,7 +470,8 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
       out[q.out] = d;
       // estimate for the agent's next search: this one's length, decaying from earlier peaks
       if (last_cost && q.cost_slot != kNoCostSlot) {
-        const uint32_t prev = last_cost[q.cost_slot], now = pops - pops0, faded = prev - (prev >> 2);
+        const uint32_t prev = last_cost[q.cost_slot], now = pops - pops0;
+        const uint32_t faded = prev == kCostUnknown ? 0u : prev - (prev >> 2);
         last_cost[q.cost_slot] = now > faded ? now : faded;
       }
     }
