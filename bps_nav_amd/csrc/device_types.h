@@ -127,8 +127,8 @@ struct alignas(16) ANode {
   float pos[3];
   float cost;
   float total;
-  uint32_t state;  // flags (1 open, 2 closed) | 1-based parent node index << 2
-  uint32_t link;   // polygon index within the scene (bits 0-14) | next node of the hash chain << 16
+  uint32_t parent;  // 1-based index of the node this one was reached from, 0 for the start node
+  uint32_t link;    // polygon index within the scene (bits 0-14) | flags (bits 15-16: 1 open, 2 closed) | next node of the hash chain << 20
   uint32_t pad;
 };
 static_assert(sizeof(ANode) == 32, "ANode");

@@ -8,7 +8,8 @@
 //   - the open list, a binary heap, in registers while it has fewer than 128 entries (entry q
 //     in lane q mod 64), then in LDS,
 //   - the hash heads of the node pool,
-//   - for the first kLinksLds nodes the hash chain link + polygon id and the flags + parent,
+//   - for the first kLinksLds nodes one word with the polygon id, the open/closed flags and the
+//     hash chain link (the parent index is read once per expansion and lives in HBM only),
 //   - the position, cost and total of the kWindow most recently created nodes (slot = index
 //     modulo kWindow); every write of those also goes to the wavefront's slot in HBM, so an
 //     older node is simply read from there.
@@ -40,7 +41,7 @@ namespace bpsx {
 #endif
 
 #ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 1024
+#define BPSX_LINKS_LDS 1536
 #endif
 #ifndef BPSX_HEAP_LDS
 #define BPSX_HEAP_LDS 128
@@ -48,7 +49,7 @@ namespace bpsx {
 #ifndef BPSX_WINDOW
 #define BPSX_WINDOW 128
 #endif
-constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link and state words are kept in LDS
+constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link word is kept in LDS
 constexpr int kHeapLds = BPSX_HEAP_LDS;     // open-list entries kept in LDS
 constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
 #ifndef BPSX_HASH
@@ -114,16 +115,18 @@ BPSX_DEV float sqrt_exact(float x) {
 // LDS of one wavefront.
 struct GeoLds {
   uint16_t first[kHashSize];
-  HeapEntry heap[kHeapLds];
-  uint32_t n_link[kLinksLds];      // polygon index (bits 0-14) | next node of the hash chain << 16
-  uint16_t n_state[kLinksLds];     // flags (1 open, 2 closed) | 1-based parent node index << 2
+  union {
+    HeapEntry heap[kHeapLds];      // open list once it has left the registers
+    uint16_t w_parent[kWindow];    // until then: 1-based parent index of the window's nodes
+  };
+  uint32_t n_link[kLinksLds];      // polygon index (bits 0-14) | flags (bits 15-16: 1 open, 2 closed) | next node of the hash chain << 20
   float w_total[kWindow];
   float w_cost[kWindow];
   float w_pos[3][kWindow];
 };
 // After A* its LDS is dead; the funnel reuses it for the corridor and its portals.  The
-// corridor is written while the nodes' links and parent indices are still being read: it lies
-// over the hash heads, which are no longer needed by then.
+// corridor is written while the nodes' links are still being read: it lies over the hash
+// heads, which are no longer needed by then.
 struct FunnelLds {
   uint16_t corridor[kMaxPath];
   uint16_t pad[kHashSize - kMaxPath];
@@ -135,11 +138,15 @@ union GeoShared {
   FunnelLds f;
 };
 
-constexpr uint32_t kChainEnd = 0xffffu;
+// One word per node holds what the search loop reads of it besides the window: the parent
+// index is needed once per expansion and for the final path, and lives in HBM only.
+constexpr uint32_t kChainEnd = 0xfffu;
+static_assert(kMaxNodes <= (int)kChainEnd, "node indices must stay below the chain end marker");
 BPSX_DEV uint32_t link_id(uint32_t l) { return l & 0x7fffu; }
-BPSX_DEV uint32_t link_next(uint32_t l) { return l >> 16; }
-BPSX_DEV uint32_t state_flags(uint32_t s) { return s & 3u; }
-BPSX_DEV uint32_t state_pidx(uint32_t s) { return s >> 2; }
+BPSX_DEV uint32_t link_flags(uint32_t l) { return (l >> 15) & 3u; }
+BPSX_DEV uint32_t link_next(uint32_t l) { return l >> 20; }
+BPSX_DEV uint32_t make_link(uint32_t id, uint32_t flags, uint32_t next) { return id | (flags << 15) | (next << 20); }
+BPSX_DEV uint32_t with_flags(uint32_t l, uint32_t flags) { return (l & ~(3u << 15)) | (flags << 15); }
 
 // Accessors take the instantiation's spill switch S: with S false every node index is below
 // kLinksLds and every heap index below kHeapLds, and no address-space branch is generated.
@@ -167,17 +174,6 @@ struct GeoWave {
     if (!S || i < kLinksLds) L->n_link[i] = v;
     else { BPSX_KEEP_APART(); ws->nodes[i].link = v; BPSX_KEEP_APART(); }
   }
-  template <bool S> BPSX_DEV uint32_t state(int i) const {
-    if (!S || i < kLinksLds) return (uint32_t)L->n_state[i];
-    BPSX_KEEP_APART();
-    const uint32_t v = ws->nodes[i].state;
-    BPSX_KEEP_APART();
-    return v;
-  }
-  template <bool S> BPSX_DEV void set_state(int i, uint32_t v) const {
-    if (!S || i < kLinksLds) L->n_state[i] = (uint16_t)v;
-    else { BPSX_KEEP_APART(); ws->nodes[i].state = v; BPSX_KEEP_APART(); }
-  }
   // node i still has its position/cost/total in LDS
   BPSX_DEV bool in_window(int i) const { return i >= nodeCount - kWindow; }
   static BPSX_DEV uint32_t hash(uint32_t ip) { return (__umul24(ip, 0x9e3779u) >> 9) & (kHashSize - 1); }
@@ -187,22 +183,25 @@ struct GeoWave {
     nodeCount = 0;
     wave_sync();
   }
-  // node index of polygon ip, or -1 (any lane, independently); one LDS access per chain step
   // Node index of polygon ip, or -1; *head receives the bucket's first node (what a new node of
-  // this bucket links to).  Called by all lanes (idle ones with valid = false): the chains are
-  // walked in step, one LDS access per lane and round, until every lane has hit or run out.
-  template <bool S> BPSX_DEV int find(bool valid, uint32_t ip, uint32_t bucket, uint32_t* head) const {
+  // this bucket links to) and *hlink the found node's link word (its flags).  Called by all
+  // lanes (idle ones with valid = false): the chains are walked in step, one LDS access per
+  // lane and round, until every lane has hit or run out.
+  template <bool S> BPSX_DEV int find(bool valid, uint32_t ip, uint32_t bucket, uint32_t* head, uint32_t* hlink) const {
     uint32_t cur = L->first[bucket];
     if (!valid) cur = kChainEnd;
     *head = cur;
     int found = -1;
+    uint32_t fl = 0;
     while (__ballot(cur != kChainEnd)) {
       const bool live = cur != kChainEnd;
       const uint32_t l = link<S>(live ? (int)cur : 0);
       const bool hit = live && link_id(l) == ip;
       found = hit ? (int)cur : found;
+      fl = hit ? l : fl;
       cur = (live && !hit) ? link_next(l) : kChainEnd;
     }
+    *hlink = fl;
     return found;
   }
 
@@ -419,13 +418,16 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     // the node about to be popped is the root: fetch its edges while the heap is repaired
     int bi;
     uint32_t bestIp;
+    uint32_t blink;   // the node's link word: closing the node rewrites its flags
     if (SH) {
       bi = uniform_i((int)L->heap[0].node);
-      bestIp = link_id((uint32_t)uniform_i((int)g.link<S>(bi)));
+      blink = g.link<S>(bi);
+      bestIp = link_id((uint32_t)uniform_i((int)blink));
     } else {
       const uint32_t root = rlane(rh.n0, 1);
       bi = (int)(root & 0x7ffu);
       bestIp = root >> 11;
+      blink = g.link<S>(bi);
     }
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
@@ -434,13 +436,17 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
     float b0, b1, b2, bcost;
+    uint32_t bparent;   // read now, moved to a scalar register only after the pop
     if (g.in_window(bi)) {
       const int w = bi & (kWindow - 1);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
+      if (!SH) bparent = L->w_parent[w];
+      else { BPSX_KEEP_APART(); bparent = g.ws->nodes[bi].parent; BPSX_KEEP_APART(); }
     } else {
       BPSX_KEEP_APART();
       const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
       b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
+      bparent = g.ws->nodes[bi].parent;
       BPSX_KEEP_APART();
 #ifdef BPSX_QUERY_TRACE
       g.missTop++;
@@ -449,13 +455,12 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
 #ifdef BPSX_QUERY_TRACE
     if (!SH && (uint32_t)rh.size > g.maxHeap) g.maxHeap = (uint32_t)rh.size;
 #endif
-    const uint32_t bstate = g.state<S>(bi);   // read now, moved to a scalar register only after the pop
     PHASE_MARK(0);
     if (SH) g.pop<true>();
     else rh.pop(lane);
-    const uint32_t pidx = state_pidx((uint32_t)uniform_i((int)bstate));
+    const uint32_t pidx = (uint32_t)uniform_i((int)bparent);
     PHASE_MARK(1);
-    g.set_state<S>(bi, 2u | (pidx << 2));   // open -> closed
+    g.set_link<S>(bi, with_flags(blink, 2u));   // open -> closed
     if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
     (*pops)++;
     // a search that runs long gets ahead of the short ones sharing its SIMD
@@ -464,8 +469,8 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
-    uint32_t chainHead;
-    int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead);
+    uint32_t chainHead, hitLink;
+    int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
     // the polygon the expanded node was reached from is not entered again
     if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
     PHASE_MARK(3);
@@ -486,11 +491,12 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       bool pending = isNew && nb != kNoNb;
       // All insert at once in front of the chain head their lookup saw.  Of several that share a
       // bucket one store wins; the others see that when they read the head back and go round
-      // again behind the winner.  One new node needs no check.
+      // again behind the winner.  One new node needs no check.  A new node is open from the
+      // start: the cost computation below always takes it.
       uint32_t head = chainHead;
       for (;;) {
         if (pending) {
-          g.set_link<S>(ni, nb | (head << 16));
+          g.set_link<S>(ni, make_link(nb, 1u, head));
           L->first[bucket] = (uint16_t)ni;
         }
         wave_sync();
@@ -508,23 +514,23 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     g.missNb += (uint32_t)__popcll(__ballot(nb != kNoNb && !isNew && !g.in_window(ni)));
 #endif
     // Costs of the step to each neighbour (lane-wise).  Written with few branches: all lanes
-    // issue the one round of LDS reads a revisited node needs (idle lanes read slot 0), the rare
-    // node that has left the window is fetched under a wave-uniform test, new nodes take the
-    // portal midpoint instead, and everything is stored in one predicated block.
+    // issue the one round of LDS reads a revisited node needs (idle lanes read slot 0; its flags
+    // came with the lookup), the rare node that has left the window is fetched under a
+    // wave-uniform test, new nodes take the portal midpoint instead, and everything is stored
+    // in one predicated block.
     const bool valid = nb != kNoNb;
     const int nis = valid ? ni : 0;
     const int w = nis & (kWindow - 1);
     const bool inw = g.in_window(nis);   // new nodes always are
     ANode& hn = g.ws->nodes[nis];
-    uint32_t fl = state_flags(g.state<S>(nis));
+    uint32_t fl = link_flags(hitLink);
     float p0 = L->w_pos[0][w], p1 = L->w_pos[1][w], p2 = L->w_pos[2][w], oldTotal = L->w_total[w];
     const bool miss = valid && !isNew && !inw;
     if (__ballot(miss)) {
       if (miss) {
         BPSX_KEEP_APART();
         const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
-        const float2 ts = *reinterpret_cast<const float2*>(&hn.total);  // total, state
-        p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = ts.x;
+        p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = hn.total;
         BPSX_KEEP_APART();
       }
     }
@@ -543,13 +549,14 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const bool update = valid && !(fl && total >= oldTotal);
     const bool wasOpen = update && (fl & 1u) != 0;
     if (update) {
-      g.set_state<S>(ni, 1u | ((uint32_t)(bi + 1) << 2));   // open, parent = expanded node
+      if (!isNew) g.set_link<S>(ni, with_flags(hitLink, 1u));   // open (again)
       if (inw) {
         L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2;   // unchanged for a revisited node
         L->w_cost[w] = cost; L->w_total[w] = total;
+        if (!SH) L->w_parent[w] = (uint16_t)(bi + 1);
       }
       *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
-      hn.total = total;
+      *reinterpret_cast<uint2*>(&hn.total) = make_uint2(__float_as_uint(total), (uint32_t)(bi + 1));   // total, parent = expanded node
     }
     wave_sync();
     PHASE_MARK(5);
@@ -621,8 +628,9 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       for (int k = 0; k < 3; ++k) { L->w_pos[k][0] = startPos[k]; hn.pos[k] = startPos[k]; }
       L->w_cost[0] = 0; L->w_total[0] = total;
       hn.cost = 0; hn.total = total;
-      L->n_state[0] = 1;   // open, no parent
-      L->n_link[0] = startIp | (kChainEnd << 16);
+      hn.parent = 0;
+      L->w_parent[0] = 0;
+      L->n_link[0] = make_link(startIp, 1u, kChainEnd);   // open
       L->first[GeoWave::hash(startIp)] = 0;
     }
     wave_sync();
@@ -648,20 +656,21 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #undef ASTAR_RUN
   (void)ex;
   const int lastBest = st.lastBest;
-  // getPathToNode
+  // getPathToNode: one walk up the parents notes the node indices (in the window's array of
+  // totals, no longer needed), then all lanes fill the corridor, which overlays the hash heads;
+  // the links stay readable while it is written
+  static_assert(sizeof(g.L->w_total) >= kMaxPath * sizeof(uint16_t), "the walk must fit the array it reuses");
+  uint16_t* walk = reinterpret_cast<uint16_t*>(g.L->w_total);
+  wave_sync();
   int length = 0;
-  for (int c = lastBest + 1; c; c = (int)state_pidx(g.state<true>(c - 1))) length++;
+  for (int c = lastBest + 1; c && length <= kMaxNodes; c = uniform_i((int)g.ws->nodes[c - 1].parent)) {
+    if (lane == 0 && length < kMaxPath) walk[length] = (uint16_t)(c - 1);
+    length++;
+  }
+  wave_sync();
   const bool ok = length <= kMaxPath && link_id(g.link<true>(lastBest)) == endIp && !st.outOfNodes;
   if (!ok) return 0;
-  // the corridor goes into LDS that overlays the nodes' cost and position arrays; the links
-  // and parent indices are outside that region and stay readable while it is written
-  if (lane == 0) {
-    int c = lastBest + 1;
-    for (int i = length - 1; i >= 0; --i) {
-      F->corridor[i] = (uint16_t)link_id(g.link<true>(c - 1));
-      c = (int)state_pidx(g.state<true>(c - 1));
-    }
-  }
+  for (int i = lane; i < length; i += 64) F->corridor[length - 1 - i] = (uint16_t)link_id(g.link<true>((int)walk[i]));
   wave_sync();
   return length;
 }
