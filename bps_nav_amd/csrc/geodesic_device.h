@@ -41,7 +41,7 @@ namespace bpsx {
 #endif
 
 #ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 1536
+#define BPSX_LINKS_LDS 1408
 #endif
 #ifndef BPSX_HEAP_LDS
 #define BPSX_HEAP_LDS 128
@@ -657,10 +657,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
   (void)ex;
   const int lastBest = st.lastBest;
   // getPathToNode: one walk up the parents notes the node indices (in the window's array of
-  // totals, no longer needed), then all lanes fill the corridor, which overlays the hash heads;
+  // positions, no longer needed), then all lanes fill the corridor, which overlays the hash heads;
   // the links stay readable while it is written
-  static_assert(sizeof(g.L->w_total) >= kMaxPath * sizeof(uint16_t), "the walk must fit the array it reuses");
-  uint16_t* walk = reinterpret_cast<uint16_t*>(g.L->w_total);
+  static_assert(sizeof(g.L->w_pos) >= kMaxPath * sizeof(uint16_t), "the walk must fit the array it reuses");
+  uint16_t* walk = reinterpret_cast<uint16_t*>(g.L->w_pos);
   wave_sync();
   int length = 0;
   for (int c = lastBest + 1; c && length <= kMaxNodes; c = uniform_i((int)g.ws->nodes[c - 1].parent)) {
