@@ -6,13 +6,13 @@
 // a shared queue when done.  The search touches almost only nodes it created recently (the
 // frontier of A* is narrow), so LDS holds what is hot and small and HBM holds the rest:
 //   - the open list, a binary heap, in registers while it has fewer than 128 entries (entry q
-//     in lane q mod 64), then in LDS,
+//     in lane q mod 64); a longer one (rare) keeps its top kHeapLds entries in LDS,
 //   - the hash heads of the node pool,
 //   - for the first kLinksLds nodes one word with the polygon id, the open/closed flags and the
 //     hash chain link (the parent index is read once per expansion and lives in HBM only),
 //   - the position, cost and total of the kWindow most recently created nodes (slot = index
-//     modulo kWindow); every write of those also goes to the wavefront's slot in HBM, so an
-//     older node is simply read from there.
+//     modulo kWindow) and their parent index; every write of those also goes to the
+//     wavefront's slot in HBM, so an older node is simply read from there.
 // Heap entries beyond kHeapLds and links beyond kLinksLds spill to the same slot.  A query
 // runs the instantiation of the loop without spill code until one more expansion could
 // outgrow the links in LDS or the register heap, then carries on in a spilling instantiation.
@@ -44,13 +44,13 @@ namespace bpsx {
 #define BPSX_LINKS_LDS 1408
 #endif
 #ifndef BPSX_HEAP_LDS
-#define BPSX_HEAP_LDS 128
+#define BPSX_HEAP_LDS 32
 #endif
 #ifndef BPSX_WINDOW
 #define BPSX_WINDOW 128
 #endif
 constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link word is kept in LDS
-constexpr int kHeapLds = BPSX_HEAP_LDS;     // open-list entries kept in LDS
+constexpr int kHeapLds = BPSX_HEAP_LDS;     // entries of an open list that has left the registers kept in LDS (its top levels)
 constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
 #ifndef BPSX_HASH
 #define BPSX_HASH 512
@@ -286,7 +286,6 @@ struct GeoWave {
 // is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
 constexpr int kRegHeap = 127;
 static_assert(kMaxNodes <= 2048, "heap entries keep the node index in 11 bits");
-static_assert(kHeapLds > kRegHeap, "the register heap must fit the LDS heap it is moved to");
 struct RegHeap {
   uint32_t t0, t1;   // total bits
   uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11, so that popping
@@ -647,8 +646,13 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     g.heapSpills++;
     // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
     const RegHeap& rh = st.rh;
-    if (lane >= 1 && lane <= rh.size) g.L->heap[lane - 1] = HeapEntry{__uint_as_float(rh.t0), rh.n0 & 0x7ffu};
-    if (64 + lane <= rh.size) g.L->heap[63 + lane] = HeapEntry{__uint_as_float(rh.t1), rh.n1 & 0x7ffu};
+    auto put = [&](int i, uint32_t t, uint32_t n) {
+      const HeapEntry e{__uint_as_float(t), n & 0x7ffu};
+      if (i < kHeapLds) g.L->heap[i] = e;
+      else { BPSX_KEEP_APART(); g.ws->heap_spill[i] = e; BPSX_KEEP_APART(); }
+    };
+    if (lane >= 1 && lane <= rh.size) put(lane - 1, rh.t0, rh.n0);
+    if (64 + lane <= rh.size) put(63 + lane, rh.t1, rh.n1);
     g.heapSize = rh.size;
     wave_sync();
     ex = ASTAR_RUN(2);
