@@ -85,8 +85,39 @@ def cpu_baseline(workload, agents_per_scene, seed, p_forward, budget_s=20.0):
         elapsed += time.perf_counter() - t0
         steps += 1
     sim.close()
+    # the same step on one thread, on a smaller sample (2 scenes), for the per-core rate
+    n1 = min(2, sample_scenes) * agents_per_scene
+    sim = bpo.Sim(lib, workload[:min(2, sample_scenes)], n1, seed=seed, threads=1)
+    sim.reset()
+    for _ in range(5):
+        sim.step(episodes.random_actions(rng, n1, p_forward))
+    steps1, elapsed1 = 0, 0.0
+    while steps1 < 200 and elapsed1 < budget_s / 4:
+        a = episodes.random_actions(rng, n1, p_forward)
+        t0 = time.perf_counter()
+        sim.step(a)
+        elapsed1 += time.perf_counter() - t0
+        steps1 += 1
+    sim.close()
     return {"value": n * steps / elapsed, "unit": "agent-steps/s", "cores": cores, "kind": lib.kind,
-            "sample": f"first {sample_scenes} of the {len(workload)} scenes, {n} agents, 20 warm-up + {steps} timed steps"}
+            "sample": f"first {sample_scenes} of the {len(workload)} scenes, {n} agents, 20 warm-up + {steps} timed steps",
+            "single_thread_value": n1 * steps1 / elapsed1,
+            "single_thread_sample": f"first 2 scenes, {n1} agents, 5 warm-up + {steps1} timed steps"}
+
+
+def measured_copy_bandwidth(torch):
+    """Bytes read plus written per second by a 256 MiB device-to-device copy on this box, in GB/s:
+    what the memory system delivers to a plain streaming kernel, next to the nominal peak."""
+    src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    return 10 * 2 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
 
 
 def main():
@@ -127,6 +158,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    copy_gbs = measured_copy_bandwidth(torch)
     gen.reset(0)
     for t in range(W):
         gen.step(0, actions[t])
@@ -159,6 +191,7 @@ def main():
     achieved = geo_bytes / K / (geo_ms * 1e-3) / 1e9 if geo_ms > 0 else 0.0
     roofline = {"bound": "hbm", "kernel": "k_geodesic", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS,
+                "measured_copy_gbs": copy_gbs, "frac_of_measured_copy": achieved / copy_gbs,
                 "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (N, S) == (16384, 128) else None,
                 "dominant_kernel_by_time": dominant,
                 "kernel_ms_per_step": kt, "algorithmic_bytes_per_step": geo_bytes / K}

@@ -149,7 +149,7 @@ BPSX_DEV void begin_reset(const NavData& nav, const AgentArrays& A, const StepPa
   store3(A.goal, gi, ep + 7);
 }
 
-__global__ __launch_bounds__(256) void k_step_move(NavData nav, AgentArrays A, StepQueues Q, StepParams P,
+__global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, StepQueues Q, StepParams P,
                                                    const int64_t* __restrict__ actions) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   bool want = false, reset = false;
@@ -562,7 +562,7 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   auto mark = [&]() { if (ev) (void)hipEventRecord(ev[e++], st); };
   mark();
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
-  hipLaunchKernelGGL(k_step_move, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P, actions_dev);
+  hipLaunchKernelGGL(k_step_move, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P, actions_dev);
   mark();
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
   mark();
