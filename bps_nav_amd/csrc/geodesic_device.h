@@ -485,7 +485,9 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         else nb = kNoNb;
       }
       const int want = g.nodeCount + count;
-      if (S && want > kMaxNodes) st.outOfNodes = true;
+      // the reference carries on without the dropped nodes, but reports anything found after
+      // that as failure (only plain DT_SUCCESS counts, PathFinder.cpp:506): the search can stop
+      if (S && want > kMaxNodes) { st.outOfNodes = true; return kAstarEmpty; }
       g.nodeCount = (!S || want < kMaxNodes) ? want : kMaxNodes;
       bool pending = isNew && nb != kNoNb;
       // All insert at once in front of the chain head their lookup saw.  Of several that share a
