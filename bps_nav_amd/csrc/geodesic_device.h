@@ -41,7 +41,7 @@ namespace bpsx {
 #endif
 
 #ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 1408
+#define BPSX_LINKS_LDS 1280
 #endif
 #ifndef BPSX_HEAP_LDS
 #define BPSX_HEAP_LDS 32
@@ -53,7 +53,7 @@ constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link word is kept in 
 constexpr int kHeapLds = BPSX_HEAP_LDS;     // entries of an open list that has left the registers kept in LDS (its top levels)
 constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
 #ifndef BPSX_HASH
-#define BPSX_HASH 512
+#define BPSX_HASH 1024
 #endif
 constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash table
 static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
