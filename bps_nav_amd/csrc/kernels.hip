@@ -352,12 +352,14 @@ __global__ __launch_bounds__(256) void k_reset_all(NavData nav, AgentArrays A, S
   if (i == 0) Q.counts[kQReset] = P.n;
 }
 
-// One wavefront per agent being reset: both snaps of the new episode, its polar observation and
-// its first geodesic query.
-__global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
-  __shared__ SnapLds lds;
+// One block of two wavefronts per agent being reset: each takes one snap of the new episode (the
+// two are independent chains of dependent loads), then the first writes the state, the polar
+// observation and the episode's first geodesic query.
+__global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
+  __shared__ SnapLds lds[2];
+  __shared__ NavPt goalPt;
   const uint32_t n = Q.counts[kQReset];
-  const int lane = (int)threadIdx.x;
+  const int lane = (int)(threadIdx.x & 63), half = (int)(threadIdx.x >> 6);
   uint32_t cands = 0;
   for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
     const uint32_t gi = Q.reset_list[i];
@@ -366,10 +368,17 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
     load3(A.pos, gi, pos);
     load3(A.goal, gi, goal);
     for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
-    const NavPt a = snap_point_wave(nav, s, pos[0], pos[1], pos[2], lds, &cands);
-    if (P.task != BPSX_TASK_POINTNAV) {
-      // no goal snap and no first query (simulator.cpp:838-843, 906-916)
-      if (lane == 0) {
+    const bool pointnav = P.task == BPSX_TASK_POINTNAV;   // the other tasks snap no goal (simulator.cpp:838-843, 906-916)
+    NavPt a{};
+    if (half == 0) a = snap_point_wave(nav, s, pos[0], pos[1], pos[2], lds[0], &cands);
+    else if (pointnav) {
+      const NavPt b = snap_point_wave(nav, s, goal[0], goal[1], goal[2], lds[1], &cands);
+      if (lane == 0) goalPt = b;
+    }
+    __syncthreads();
+    if (!pointnav) {
+      // no first query either
+      if (threadIdx.x == 0) {
         const float axyz[3] = {a.x, a.y, a.z}, zero[3] = {0, 0, 0};
         store3(A.nav_xyz, gi, axyz);
         A.nav_ref[gi] = a.ref;
@@ -387,10 +396,8 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
           visit_cell(A, gi, pos);
         }
       }
-      continue;
-    }
-    const NavPt b = snap_point_wave(nav, s, goal[0], goal[1], goal[2], lds, &cands);
-    if (lane == 0) {
+    } else if (threadIdx.x == 0) {
+      const NavPt b = goalPt;
       const float axyz[3] = {a.x, a.y, a.z}, bxyz[3] = {b.x, b.y, b.z};
       store3(A.nav_xyz, gi, axyz);
       A.nav_ref[gi] = a.ref;
@@ -407,8 +414,9 @@ __global__ __launch_bounds__(64) void k_reset_snap(NavData nav, AgentArrays A, S
       // a new episode: no history
       Q.queries[(size_t)kGeoClassUnknown * Q.stride + atomicAdd(&Q.counts[kQGeo + kGeoClassUnknown], 1u)] = q;
     }
+    __syncthreads();   // goalPt is rewritten in the next round
   }
-  if (lane == 0 && blockIdx.x == 0 && n) atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
+  if (threadIdx.x == 0 && blockIdx.x == 0 && n) atomicAdd((unsigned long long*)&P.counters[kCntResets], (unsigned long long)n);
   if (lane == 0 && cands) atomicAdd((unsigned long long*)&P.counters[kCntSnapCands], (unsigned long long)cands);
 }
 
@@ -564,7 +572,7 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
   hipLaunchKernelGGL(k_step_move, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P, actions_dev);
   mark();
-  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
+  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, P);
   mark();
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, A.last_cost, slots, geo_blocks,
                   P.counters, st);
@@ -577,7 +585,7 @@ void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q,
                   uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st) {
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
   hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
-  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(64), 0, st, nav, A, Q, P);
+  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, P);
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, A.last_cost, slots, geo_blocks,
                   P.counters, st);
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
