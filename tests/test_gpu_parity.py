@@ -336,18 +336,19 @@ def test_mixed_scenes_at_the_largest_configured_shape(oracle, torch_cuda):
 
 
 def test_full_size_workload_properties(oracle, torch_cuda):
-    """The benchmark's own shape (16384 agents, 128 maze scenes of ~30k polygons), where the
-    oracle cannot step along: size-independent properties plus oracle spot checks.
+    """The benchmark's own shape (16384 agents, 128 maze scenes of ~30k polygons):
+    size-independent properties, oracle spot checks, and the oracle stepped along on all host cores.
       - every finite distance is at least the straight line between its two navmesh points;
       - rewards obey the reference's algebra given the infos (simulator.cpp:800-825);
       - a sample of agents' distances equals the oracle's geodesic for the same two points;
-      - a second simulator with the same seed produces bit-identical outputs."""
+      - a second simulator with the same seed produces bit-identical outputs;
+      - after the same steps the oracle holds the same polygon ids, positions, dones and infos, bit for bit."""
     import torch
     from bps_nav_amd import episodes, scenes
     from bps_nav_amd.bps_sim import PointNavRolloutGenerator, nav_only
     from oracle import bpo
     print("case: full-size workload properties", flush=True)
-    N, S, steps = 16384, 128, 12
+    N, S, steps = 16384, 128, 40
     blobs = [scenes.config_scene(4, i) for i in range(S)]
     nav = nav_only(blobs)
 
@@ -408,6 +409,20 @@ def test_full_size_workload_properties(oracle, torch_cuda):
         assert fresh.sum() > 8
         assert np.array_equal(common.bits(want), common.bits(r["info"][ids][fresh, 2])), "distance differs from the oracle's"
         onav.close()
+    # the oracle on the same scenes, episodes, seed and actions: a difference at any earlier step persists
+    import os
+    cpu = bpo.Sim(oracle, sc, N, seed=77, threads=min(16, len(os.sched_getaffinity(0))))
+    cpu.reset()
+    for a in acts:
+        cpu.step(a)
+    co, cs = cpu.outputs(), cpu.state()
+    cpu.close()
+    assert np.array_equal(cs["poly_ref"], r["ref"].view(np.uint32)), "polygon ids differ from the oracle's"
+    assert np.array_equal(common.bits(cs["position"]), common.bits(r["pos"])), "positions differ from the oracle's"
+    assert np.array_equal(co["masks"], r["mask"]), "dones differ from the oracle's"
+    same = common.bits(co["infos"]) == common.bits(r["info"])
+    assert (same | np.isnan(r["info"])).all(), "infos differ from the oracle's"
+    np.testing.assert_allclose(r["rew"], co["rewards"], rtol=1e-3, atol=1e-6, equal_nan=True)
     # straight-line bound, all agents: geodesic(goal point -> agent) >= |goal - agent| (3-D), using rho of the polar
     d = r["info"][:, 2]
     assert np.isfinite(d).mean() > 0.99
