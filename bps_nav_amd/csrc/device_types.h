@@ -160,8 +160,8 @@ constexpr uint32_t kNoCostSlot = 0xffffffffu;
 // Path searches differ in length by two orders of magnitude and each is sequential, so a step
 // ends when its longest search ends.  Queries are therefore queued in classes of expected
 // cost (the nodes the agent's previous searches expanded) and served from the longest class
-// down, which approximates longest-first scheduling; a search that runs long also raises its
-// wavefront's issue priority.
+// down, which approximates longest-first scheduling; the longer classes also run at a higher
+// issue priority of their wavefront.
 constexpr int kGeoClasses = 16;
 constexpr uint32_t kGeoClassWidth = 100;   // expanded nodes per class: 1500 and more, 1400-1499, ..., below 100
 constexpr __host__ __device__ uint32_t geo_class(uint32_t last_cost) {

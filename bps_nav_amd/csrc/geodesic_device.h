@@ -157,7 +157,6 @@ struct GeoWave {
   int heapSize;
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
-  int basePrio;                      // issue priority the query started with
 #ifdef BPSX_QUERY_TRACE
   uint32_t missTop, missNb, maxHeap;
 #endif
@@ -390,7 +389,6 @@ struct AstarState {
   int lastBest;
   float lastBestCost;
   bool outOfNodes;
-  int expanded;
   RegHeap rh;
 };
 enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
@@ -462,10 +460,6 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     g.set_link<S>(bi, with_flags(blink, 2u));   // open -> closed
     if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
     (*pops)++;
-    // a search that runs long gets ahead of the short ones sharing its SIMD
-    if ((++st.expanded & 255) == 0) {
-      set_wave_priority(g.basePrio + (st.expanded >> 8));
-    }
     PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
     uint32_t chainHead, hitLink;
@@ -638,7 +632,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.lastBest = 0;
     st.lastBestCost = total;
     st.outOfNodes = false;
-    st.expanded = 0;
     st.rh.init();
     st.rh.push(__float_as_uint(total), startIp << 11, lane);
   }

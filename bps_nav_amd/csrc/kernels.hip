@@ -459,8 +459,7 @@ __global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __
     g.missTop = g.missNb = g.maxHeap = 0;
     const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
-    g.basePrio = (kGeoClasses - 1 - cls) >> 2;
-    set_wave_priority(g.basePrio);
+    set_wave_priority((kGeoClasses - 1 - cls) >> 2);   // the longer the expected search, the sooner its instructions issue
 #ifdef BPSX_PHASE_TIMING
     const float d = geodesic_query(g, nav, q, &pops, &corridor, phase_acc);
 #else
