@@ -406,6 +406,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
   GeoLds* L = g.L;
   const float H_SCALE = 0.999f;
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
+  endIp = (uint32_t)uniform_i((int)endIp);   // the same in all lanes: the goal test stays on the scalar unit
   constexpr bool S = M >= 1;    // links and states may be in HBM
   constexpr bool SH = M == 2;   // open list in LDS/HBM
   RegHeap& rh = st.rh;
