@@ -314,24 +314,24 @@ int bpsx_finalize(bpsx_sim* sim) {
     HIP_TRY(hipMemcpy(A.rot, rot.data(), N * 16, hipMemcpyHostToDevice));
   }
   if ((rc = sim->alloc(&sim->d_error, 1)) || (rc = sim->alloc(&sim->d_counters, BPSX_NUM_COUNTERS))) return rc;
-  if ((rc = sim->alloc(&sim->d_batch_counts, kGeoClasses + 1))) return rc;
+  if ((rc = sim->alloc(&sim->d_batch_counts, kGeoClasses + 2))) return rc;
 
   // ---- A* wavefronts: as many as the LDS of the device holds at once, not one per agent
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, sim->cfg.gpu_id));
-  uint32_t per_cu = geodesic_blocks_per_cu();
-  if (const char* e = getenv("BPSX_GEO_WAVES_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e));
+  uint32_t per_cu = geodesic_blocks_per_cu();   // blocks of two wavefronts
+  if (const char* e = getenv("BPSX_GEO_WAVES_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e) / 2);
   uint32_t blocks = (uint32_t)prop.multiProcessorCount * per_cu;
-  if (blocks > 2 * sim->envs_per_group) blocks = 2 * sim->envs_per_group;
+  if (blocks > sim->envs_per_group) blocks = sim->envs_per_group;
   sim->geo_blocks = std::max(1u, blocks);
   sim->snap_blocks = std::max(1u, std::min((uint32_t)prop.multiProcessorCount * 16u, sim->envs_per_group));
-  if ((rc = sim->alloc(&sim->d_slots, (size_t)sim->geo_blocks))) return rc;
+  if ((rc = sim->alloc(&sim->d_slots, (size_t)sim->geo_blocks * 2))) return rc;   // one per wavefront
 
   // ---- per-group queues
   sim->groups.resize(sim->num_groups);
   const size_t n = sim->envs_per_group;
   for (auto& g : sim->groups) {
-    if ((rc = sim->alloc(&g.Q.counts, kGeoClasses + 2)) || (rc = sim->alloc(&g.Q.queries, (size_t)kGeoClasses * 2 * n)) ||
+    if ((rc = sim->alloc(&g.Q.counts, kQCounters)) || (rc = sim->alloc(&g.Q.queries, (size_t)kGeoClasses * 2 * n)) ||
         (rc = sim->alloc(&g.Q.reset_list, n)) || (rc = sim->alloc(&g.d_actions, n)))
       return rc;
     g.Q.stride = (uint32_t)(2 * n);

@@ -27,9 +27,15 @@
 // Reference semantics followed: DetourNavMeshQuery.cpp:945-1178 (findPath, getPathToNode),
 // :1661-1696, 1765-1994 (appendVertex, findStraightPath), :2279-2381 (getPortalPoints,
 // getEdgeMidPoint); DetourNode.cpp:50-200 (node pool, heap order); PathFinder.cpp:473-541.
-#pragma once
+//
+// The sizes of the LDS structures are build parameters (BPSX_LINKS_LDS, BPSX_HEAP_LDS,
+// BPSX_WINDOW, BPSX_HASH), and everything that depends on them lives in namespace
+// bpsx::BPSX_GEO_NS (default geo): the file can be included again with other values and
+// another namespace name to get a second instantiation of the same search.
 #include "nav_device.h"
 
+#ifndef BPSX_GEODESIC_COMMON_H
+#define BPSX_GEODESIC_COMMON_H
 namespace bpsx {
 
 #ifdef BPSX_ASM_MARKS
@@ -39,24 +45,6 @@ namespace bpsx {
 #else
 #define PHASE_MARK(k) do { } while (0)
 #endif
-
-#ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 1280
-#endif
-#ifndef BPSX_HEAP_LDS
-#define BPSX_HEAP_LDS 32
-#endif
-#ifndef BPSX_WINDOW
-#define BPSX_WINDOW 128
-#endif
-constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link word is kept in LDS
-constexpr int kHeapLds = BPSX_HEAP_LDS;     // entries of an open list that has left the registers kept in LDS (its top levels)
-constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
-#ifndef BPSX_HASH
-#define BPSX_HASH 1024
-#endif
-constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash table
-static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
 
 BPSX_DEV void wave_sync() {
   // All lanes belong to one wavefront: LDS and memory operations issue in program order, so
@@ -112,6 +100,169 @@ BPSX_DEV float sqrt_exact(float x) {
   return r;
 }
 
+// One word per node holds what the search loop reads of it besides the window: the parent
+// index is needed once per expansion and for the final path, and lives in HBM only.
+constexpr uint32_t kChainEnd = 0xfffu;
+static_assert(kMaxNodes <= (int)kChainEnd, "node indices must stay below the chain end marker");
+BPSX_DEV uint32_t link_id(uint32_t l) { return l & 0x7fffu; }
+BPSX_DEV uint32_t link_flags(uint32_t l) { return (l >> 15) & 3u; }
+BPSX_DEV uint32_t link_next(uint32_t l) { return l >> 20; }
+BPSX_DEV uint32_t make_link(uint32_t id, uint32_t flags, uint32_t next) { return id | (flags << 15) | (next << 20); }
+BPSX_DEV uint32_t with_flags(uint32_t l, uint32_t flags) { return (l & ~(3u << 15)) | (flags << 15); }
+
+// The open list in registers.  Heap position q (1-based, root = 1; the reference's index + 1)
+// lives in lane q & 63 of the first register pair (q < 64) or of the second (64 <= q < 128).
+// Totals are kept as bit patterns and compared as unsigned integers: they are sums of
+// distances, never negative and never NaN, and for such floats the integer order of the bits
+// is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
+constexpr int kRegHeap = 127;
+static_assert(kMaxNodes <= 2048, "heap entries keep the node index in 11 bits");
+struct RegHeap {
+  uint32_t t0, t1;   // total bits
+  uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11, so that popping
+                     // the root names the edge records to fetch without a detour through LDS
+  int size;
+  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
+  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
+  static BPSX_DEV uint32_t xlane(int src_lane, uint32_t v) {   // v of another lane; all lanes must be active
+    return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane * 4, (int)v);
+  }
+
+  // dtNodeQueue::bubbleUp of entry (t, n) from position q, by all lanes at once.  The lanes on
+  // the way from q to the root read their parent's entry; ancestors with a greater key move
+  // one step down that way (they form a run from q upwards: keys never increase towards the
+  // root) and the entry lands on top of the run.  Positions 64..127 have all their ancestors
+  // in the first pair, so only q itself can be in the second.
+  BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n, int lane) {
+    const int up = (31 - __clz(q)) - (31 - __clz(lane));   // lane 0 (clz 32) is no heap position
+    const bool on = lane >= 1 && up >= 0 && (q >> (up & 31)) == lane;
+    const uint32_t pk = xlane(lane >> 1, t0), pn = xlane(lane >> 1, n0);
+    const bool parentMoves = on && lane > 1 && pk > t;
+    const bool vacant = lane == q || t0 > t;
+    const bool land = on && vacant && !parentMoves;
+    if (q >= 64) {
+      const uint32_t qk = rlane(t0, q >> 1), qn = rlane(n0, q >> 1);
+      const bool here = lane == (q & 63);
+      t1 = here ? (qk > t ? qk : t) : t1;
+      n1 = here ? (qk > t ? qn : n) : n1;
+    }
+    t0 = parentMoves ? pk : (land ? t : t0);
+    n0 = parentMoves ? pn : (land ? n : n0);
+  }
+  BPSX_DEV void push(uint32_t t, uint32_t n, int lane) {
+    size++;
+    bubble_up(size, t, n, lane);
+  }
+  // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
+  BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
+    const unsigned long long m0 = __ballot(lane >= 1 && lane <= size && n0 == n);
+    const unsigned long long m1 = m0 ? 0ull : __ballot(64 + lane <= size && n1 == n);
+    if (!(m0 | m1)) return;
+    const int q = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
+    bubble_up(q, t, n, lane);
+  }
+  // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
+  // by the root down to a leaf along the smaller children and then bubbles the former last
+  // entry up from there; along that route keys never decrease, so the entry ends up above
+  // the first route element greater than it and nothing below moves.  Which child the hole
+  // moves to depends only on the children's keys, which the moves above them do not change:
+  // every lane q picks the smaller child of position q (cross-lane reads; positions past the
+  // end hold kEmpty), the route is read off that table with dependent lane reads, and then
+  // every route position whose smaller child is not greater than the entry takes that child,
+  // and the first one whose child is greater takes the entry.
+  BPSX_DEV void pop(int lane) {
+    const int last = size;
+    size--;
+    uint32_t lt, ln;
+    if (last < 64) { lt = rlane(t0, last); ln = rlane(n0, last); t0 = wlane(t0, kEmpty, last); }
+    else { lt = rlane(t1, last & 63); ln = rlane(n1, last & 63); t1 = wlane(t1, kEmpty, last & 63); }
+    if (size == 0) return;
+    const bool wide = size >= 64;           // entries in the second pair
+    const bool lo = lane < 32;              // children of positions 32..63 are in the second pair
+    const int c0 = (2 * lane) & 63;
+    // keys and nodes of both children in one round of cross-lane reads
+    uint32_t cl = xlane(c0, t0), cr = xlane(c0 + 1, t0);
+    uint32_t nl = xlane(c0, n0), nr = xlane(c0 + 1, n0);
+    if (wide) {
+      const uint32_t hl = xlane(c0, t1), hr = xlane(c0 + 1, t1), ml = xlane(c0, n1), mr = xlane(c0 + 1, n1);
+      cl = lo ? cl : hl; cr = lo ? cr : hr; nl = lo ? nl : ml; nr = lo ? nr : mr;
+    } else {
+      cl = lo ? cl : kEmpty; cr = lo ? cr : kEmpty;
+    }
+    const bool right = cr < cl;
+    const uint32_t cmin = right ? cr : cl;
+    const uint32_t cn = right ? nr : nl;
+    const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);   // position 2..127
+    // route of the hole: 1, choice[1], choice[choice[1]], ...
+    unsigned long long route = 2ull;
+    uint32_t q = 1;
+#pragma unroll
+    for (int lvl = 0; lvl < 5; ++lvl) {
+      q = rlane(choice, (int)(q & 31));     // levels 0..4 start from positions below 32
+      route |= 1ull << (q & 63);
+    }
+    const bool on = (route >> lane) & 1ull;
+    const bool take = on && cmin <= lt;
+    const bool land = on && !take && (lane == 1 || t0 <= lt);
+    if (wide) {
+      // sixth level: from position q in 32..63 to its smaller child in the second pair, which has
+      // no children of its own: it takes the entry if its parent took it
+      const uint32_t e = rlane(choice, (int)(q & 63));
+      const bool here = lane == (int)(e & 63) && t1 <= lt;
+      t1 = here ? lt : t1;
+      n1 = here ? ln : n1;
+    }
+    t0 = take ? cmin : (land ? lt : t0);
+    n0 = take ? cn : (land ? ln : n0);
+  }
+};
+
+struct AstarState {
+  int lastBest;
+  float lastBestCost;
+  bool outOfNodes;
+  RegHeap rh;
+};
+enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
+
+BPSX_DEV float tri_area2d(const float* a, const float* b, const float* c) {
+  const float abx = b[0] - a[0], abz = b[2] - a[2];
+  const float acx = c[0] - a[0], acz = c[2] - a[2];
+  return acx * abz - abx * acz;
+}
+BPSX_DEV bool vequal(const float* a, const float* b) {
+  const float thr = (1.0f / 16384.0f) * (1.0f / 16384.0f);
+  const float dx = b[0] - a[0], dy = b[1] - a[1], dz = b[2] - a[2];
+  return dx * dx + dy * dy + dz * dz < thr;
+}
+
+}  // namespace bpsx
+#endif  // BPSX_GEODESIC_COMMON_H
+
+#ifndef BPSX_GEO_NS
+#define BPSX_GEO_NS geo
+#endif
+namespace bpsx {
+namespace BPSX_GEO_NS {
+
+#ifndef BPSX_LINKS_LDS
+#define BPSX_LINKS_LDS 1152
+#endif
+#ifndef BPSX_HEAP_LDS
+#define BPSX_HEAP_LDS 32
+#endif
+#ifndef BPSX_WINDOW
+#define BPSX_WINDOW 128
+#endif
+constexpr int kLinksLds = BPSX_LINKS_LDS;   // nodes whose link word is kept in LDS
+constexpr int kHeapLds = BPSX_HEAP_LDS;     // entries of an open list that has left the registers kept in LDS (its top levels)
+constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/cost/total are kept in LDS
+#ifndef BPSX_HASH
+#define BPSX_HASH 512
+#endif
+constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash table
+static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
+
 // LDS of one wavefront.
 struct GeoLds {
   uint16_t first[kHashSize];
@@ -137,16 +288,6 @@ union GeoShared {
   GeoLds a;
   FunnelLds f;
 };
-
-// One word per node holds what the search loop reads of it besides the window: the parent
-// index is needed once per expansion and for the final path, and lives in HBM only.
-constexpr uint32_t kChainEnd = 0xfffu;
-static_assert(kMaxNodes <= (int)kChainEnd, "node indices must stay below the chain end marker");
-BPSX_DEV uint32_t link_id(uint32_t l) { return l & 0x7fffu; }
-BPSX_DEV uint32_t link_flags(uint32_t l) { return (l >> 15) & 3u; }
-BPSX_DEV uint32_t link_next(uint32_t l) { return l >> 20; }
-BPSX_DEV uint32_t make_link(uint32_t id, uint32_t flags, uint32_t next) { return id | (flags << 15) | (next << 20); }
-BPSX_DEV uint32_t with_flags(uint32_t l, uint32_t flags) { return (l & ~(3u << 15)) | (flags << 15); }
 
 // Accessors take the instantiation's spill switch S: with S false every node index is below
 // kLinksLds and every heap index below kHeapLds, and no address-space branch is generated.
@@ -277,121 +418,6 @@ struct GeoWave {
     wave_sync();
   }
 };
-
-// The open list in registers.  Heap position q (1-based, root = 1; the reference's index + 1)
-// lives in lane q & 63 of the first register pair (q < 64) or of the second (64 <= q < 128).
-// Totals are kept as bit patterns and compared as unsigned integers: they are sums of
-// distances, never negative and never NaN, and for such floats the integer order of the bits
-// is the float order.  Same algorithm as dtNodeQueue (DetourNode.cpp:150-200).
-constexpr int kRegHeap = 127;
-static_assert(kMaxNodes <= 2048, "heap entries keep the node index in 11 bits");
-struct RegHeap {
-  uint32_t t0, t1;   // total bits
-  uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11, so that popping
-                     // the root names the edge records to fetch without a detour through LDS
-  int size;
-  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
-  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
-  static BPSX_DEV uint32_t xlane(int src_lane, uint32_t v) {   // v of another lane; all lanes must be active
-    return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane * 4, (int)v);
-  }
-
-  // dtNodeQueue::bubbleUp of entry (t, n) from position q, by all lanes at once.  The lanes on
-  // the way from q to the root read their parent's entry; ancestors with a greater key move
-  // one step down that way (they form a run from q upwards: keys never increase towards the
-  // root) and the entry lands on top of the run.  Positions 64..127 have all their ancestors
-  // in the first pair, so only q itself can be in the second.
-  BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n, int lane) {
-    const int up = (31 - __clz(q)) - (31 - __clz(lane));   // lane 0 (clz 32) is no heap position
-    const bool on = lane >= 1 && up >= 0 && (q >> (up & 31)) == lane;
-    const uint32_t pk = xlane(lane >> 1, t0), pn = xlane(lane >> 1, n0);
-    const bool parentMoves = on && lane > 1 && pk > t;
-    const bool vacant = lane == q || t0 > t;
-    const bool land = on && vacant && !parentMoves;
-    if (q >= 64) {
-      const uint32_t qk = rlane(t0, q >> 1), qn = rlane(n0, q >> 1);
-      const bool here = lane == (q & 63);
-      t1 = here ? (qk > t ? qk : t) : t1;
-      n1 = here ? (qk > t ? qn : n) : n1;
-    }
-    t0 = parentMoves ? pk : (land ? t : t0);
-    n0 = parentMoves ? pn : (land ? n : n0);
-  }
-  BPSX_DEV void push(uint32_t t, uint32_t n, int lane) {
-    size++;
-    bubble_up(size, t, n, lane);
-  }
-  // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
-  BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
-    const unsigned long long m0 = __ballot(lane >= 1 && lane <= size && n0 == n);
-    const unsigned long long m1 = m0 ? 0ull : __ballot(64 + lane <= size && n1 == n);
-    if (!(m0 | m1)) return;
-    const int q = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
-    bubble_up(q, t, n, lane);
-  }
-  // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
-  // by the root down to a leaf along the smaller children and then bubbles the former last
-  // entry up from there; along that route keys never decrease, so the entry ends up above
-  // the first route element greater than it and nothing below moves.  Which child the hole
-  // moves to depends only on the children's keys, which the moves above them do not change:
-  // every lane q picks the smaller child of position q (cross-lane reads; positions past the
-  // end hold kEmpty), the route is read off that table with dependent lane reads, and then
-  // every route position whose smaller child is not greater than the entry takes that child,
-  // and the first one whose child is greater takes the entry.
-  BPSX_DEV void pop(int lane) {
-    const int last = size;
-    size--;
-    uint32_t lt, ln;
-    if (last < 64) { lt = rlane(t0, last); ln = rlane(n0, last); t0 = wlane(t0, kEmpty, last); }
-    else { lt = rlane(t1, last & 63); ln = rlane(n1, last & 63); t1 = wlane(t1, kEmpty, last & 63); }
-    if (size == 0) return;
-    const bool wide = size >= 64;           // entries in the second pair
-    const bool lo = lane < 32;              // children of positions 32..63 are in the second pair
-    const int c0 = (2 * lane) & 63;
-    // keys and nodes of both children in one round of cross-lane reads
-    uint32_t cl = xlane(c0, t0), cr = xlane(c0 + 1, t0);
-    uint32_t nl = xlane(c0, n0), nr = xlane(c0 + 1, n0);
-    if (wide) {
-      const uint32_t hl = xlane(c0, t1), hr = xlane(c0 + 1, t1), ml = xlane(c0, n1), mr = xlane(c0 + 1, n1);
-      cl = lo ? cl : hl; cr = lo ? cr : hr; nl = lo ? nl : ml; nr = lo ? nr : mr;
-    } else {
-      cl = lo ? cl : kEmpty; cr = lo ? cr : kEmpty;
-    }
-    const bool right = cr < cl;
-    const uint32_t cmin = right ? cr : cl;
-    const uint32_t cn = right ? nr : nl;
-    const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);   // position 2..127
-    // route of the hole: 1, choice[1], choice[choice[1]], ...
-    unsigned long long route = 2ull;
-    uint32_t q = 1;
-#pragma unroll
-    for (int lvl = 0; lvl < 5; ++lvl) {
-      q = rlane(choice, (int)(q & 31));     // levels 0..4 start from positions below 32
-      route |= 1ull << (q & 63);
-    }
-    const bool on = (route >> lane) & 1ull;
-    const bool take = on && cmin <= lt;
-    const bool land = on && !take && (lane == 1 || t0 <= lt);
-    if (wide) {
-      // sixth level: from position q in 32..63 to its smaller child in the second pair, which has
-      // no children of its own: it takes the entry if its parent took it
-      const uint32_t e = rlane(choice, (int)(q & 63));
-      const bool here = lane == (int)(e & 63) && t1 <= lt;
-      t1 = here ? lt : t1;
-      n1 = here ? ln : n1;
-    }
-    t0 = take ? cmin : (land ? lt : t0);
-    n0 = take ? cn : (land ? ln : n0);
-  }
-};
-
-struct AstarState {
-  int lastBest;
-  float lastBestCost;
-  bool outOfNodes;
-  RegHeap rh;
-};
-enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
 
 // The expansion loop of findPath.  M = 0: open list in registers, all links in LDS; M = 1: open
 // list in registers, links may spill; M = 2: open list in LDS/HBM, links may spill.  Returns
@@ -675,17 +701,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
   return length;
 }
 
-BPSX_DEV float tri_area2d(const float* a, const float* b, const float* c) {
-  const float abx = b[0] - a[0], abz = b[2] - a[2];
-  const float acx = c[0] - a[0], acz = c[2] - a[2];
-  return acx * abz - abx * acz;
-}
-BPSX_DEV bool vequal(const float* a, const float* b) {
-  const float thr = (1.0f / 16384.0f) * (1.0f / 16384.0f);
-  const float dx = b[0] - a[0], dy = b[1] - a[1], dz = b[2] - a[2];
-  return dx * dx + dy * dy + dz * dz < thr;
-}
-
 // String pulling over F->corridor[0..n) and the summed length; +inf for every outcome the
 // reference maps to "no path" (straight path of 256 points or more, missing portal).
 BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const SceneDev& s, int n, const float* startPos,
@@ -818,4 +833,5 @@ BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q,
   return len;
 }
 
+}  // namespace BPSX_GEO_NS
 }  // namespace bpsx

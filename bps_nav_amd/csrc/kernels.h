@@ -6,11 +6,11 @@
 
 namespace bpsx {
 
-enum QueueCounter { kQGeo = 0 /* one per cost class */, kQGeoHead = kGeoClasses, kQReset };
+enum QueueCounter { kQGeo = 0 /* one per cost class */, kQGeoHead = kGeoClasses, kQReset, kQGeoHeadLong, kQCounters };
 
 // Work queues of one step, all in HBM, sized for every agent of a group.
 struct StepQueues {
-  uint32_t* counts;          // [kGeoClasses + 2], see QueueCounter
+  uint32_t* counts;          // [kQCounters], see QueueCounter
   GeoQuery* queries;         // [kGeoClasses][stride]: one per moved/finished agent plus one per reset
   uint32_t stride;           // 2n
   uint32_t* reset_list;      // [n] agent indices being reset
@@ -48,7 +48,7 @@ void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uin
 void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
                            uint32_t n, float* oxyz, uint32_t* oref, hipStream_t st);
 void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
-                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 1] */,
+                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 2] */,
                            float* out,
                            GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st);
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,

@@ -20,6 +20,23 @@
 
 #include "../../include/bpsx.h"
 #include "geodesic_device.h"
+// A second instantiation of the same search for the few longest queries of a step: all 2048
+// link words, twice the window and twice the hash heads in LDS.  Such a query takes the LDS of a
+// whole two-wavefront block (see k_geodesic).
+#undef BPSX_GEO_NS
+#undef BPSX_LINKS_LDS
+#undef BPSX_HEAP_LDS
+#undef BPSX_WINDOW
+#undef BPSX_HASH
+#define BPSX_GEO_NS geo_long
+#define BPSX_LINKS_LDS 2048
+#define BPSX_HEAP_LDS 32
+#define BPSX_WINDOW 256
+#ifndef BPSX_LONG_HASH
+#define BPSX_LONG_HASH 1024
+#endif
+#define BPSX_HASH BPSX_LONG_HASH
+#include "geodesic_device.h"
 #include "kernels.h"
 
 namespace bpsx {
@@ -113,7 +130,7 @@ BPSX_DEV uint32_t visit_cell(const AgentArrays& A, uint32_t gi, const float* pos
 __global__ void k_clear_queues(StepQueues Q) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     for (int c = 0; c < kGeoClasses; ++c) Q.counts[kQGeo + c] = 0;
-    Q.counts[kQGeoHead] = 0; Q.counts[kQReset] = 0;
+    Q.counts[kQGeoHead] = 0; Q.counts[kQGeoHeadLong] = 0; Q.counts[kQReset] = 0;
   }
 }
 
@@ -425,74 +442,121 @@ __global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, 
 __device__ unsigned long long g_trace[1 << 17][4];
 __device__ unsigned int g_trace_n;
 #endif
-__global__ __launch_bounds__(64) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
-                                                 const uint32_t* __restrict__ counts, uint32_t* head, float* out,
-                                                 uint32_t* last_cost, GeoSlot* slots, uint64_t* counters) {
-  __shared__ GeoShared lds;
-  GeoWave g;
-  g.lane = (int)threadIdx.x;
-  g.L = &lds.a;
-  g.ws = &slots[blockIdx.x];
-  g.heapSize = 0;
-  g.nodeCount = 0;
-  g.linkSpills = g.heapSpills = 0;
-  // classes are served in order: class c owns ticket numbers [first[c], first[c + 1])
-  uint32_t first[kGeoClasses + 1];
-  first[0] = 0;
-  for (int c = 0; c < kGeoClasses; ++c) first[c + 1] = first[c] + (uint32_t)uniform_i((int)counts[c]);
-  const uint32_t nq = first[kGeoClasses];
+// Work of one wavefront on one query, whichever instantiation g belongs to: the search, the
+// result and the agent's cost estimate.
+struct GeoTotals {
   uint32_t pops = 0, corridor = 0, done = 0;
 #ifdef BPSX_PHASE_TIMING
   unsigned long long phase_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #endif
+};
+template <class Wave>
+BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cls, float* out, uint32_t* last_cost, GeoTotals& T) {
+  const uint32_t pops0 = T.pops;
+#ifdef BPSX_QUERY_TRACE
+  const unsigned long long trace_t0 = wall_clock64();
+  g.missTop = g.missNb = g.maxHeap = 0;
+  const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
+#endif
+  // the longer the expected search, the sooner its instructions issue; a search of unknown
+  // length may be among the longest
+  set_wave_priority(cls == (int)kGeoClassUnknown ? 3 : (kGeoClasses - 1 - cls) >> 2);
+#ifdef BPSX_PHASE_TIMING
+  const float d = geodesic_query(g, nav, q, &T.pops, &T.corridor, T.phase_acc);
+#else
+  const float d = geodesic_query(g, nav, q, &T.pops, &T.corridor);
+#endif
+  if (g.lane == 0) {
+#ifdef BPSX_QUERY_TRACE
+    const unsigned int ti = atomicAdd(&g_trace_n, 1u);
+    if (ti < (1u << 17)) {
+      g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = T.pops - pops0;
+      g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)(g.missTop & 0xfffu) << 24) |
+                        ((unsigned long long)(g.missNb & 0xfffu) << 36) | ((unsigned long long)(g.maxHeap & 0xffu) << 48);
+    }
+#endif
+    out[q.out] = d;
+    // estimate for the agent's next search: this one's length, decaying from earlier peaks
+    if (last_cost && q.cost_slot != kNoCostSlot) {
+      const uint32_t prev = last_cost[q.cost_slot], now = T.pops - pops0;
+      const uint32_t faded = prev == kCostUnknown ? 0u : prev - (prev >> 2);
+      last_cost[q.cost_slot] = now > faded ? now : faded;
+    }
+  }
+  T.done++;
+  wave_sync();
+}
+
+// Blocks of two wavefronts, each wavefront persistent and serving queries from the shared
+// queue on its half of the block's LDS.  The launch ends with its longest search, so the
+// queries of the kLongClasses longest classes are treated apart: at its start the first
+// wavefront of every block draws a ticket for one of them, and a block that gets one gives it
+// the whole block's LDS (the larger instantiation: no link spills, half the window misses,
+// shorter hash chains; 7 % faster on such searches) while its second wavefront leaves.
+constexpr int kLongClasses = 2;   // expected cost of 1400 nodes and more
+__global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
+                                                  const uint32_t* __restrict__ counts, uint32_t* head, uint32_t* head_long,
+                                                  float* out, uint32_t* last_cost, GeoSlot* slots, uint64_t* counters) {
+  constexpr size_t kHalf = sizeof(geo::GeoShared);
+  static_assert(kHalf % 16 == 0 && sizeof(geo_long::GeoShared) <= 2 * kHalf, "the long search must fit the LDS of one block");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kHalf];
+  __shared__ uint32_t long_ticket;
+  const int lane = (int)(threadIdx.x & 63), half = (int)(threadIdx.x >> 6);
+  GeoSlot* slot = &slots[blockIdx.x * 2 + half];
+  // classes are served in order: class c owns ticket numbers [first[c], first[c + 1])
+  uint32_t first[kGeoClasses + 1];
+  first[0] = 0;
+  for (int c = 0; c < kGeoClasses; ++c) first[c + 1] = first[c] + (uint32_t)uniform_i((int)counts[c]);
+  const uint32_t nq = first[kGeoClasses], nlong = first[kLongClasses];
+  GeoTotals T;
+  uint32_t linkSpills = 0, heapSpills = 0;
+  if (threadIdx.x == 0) long_ticket = atomicAdd(head_long, 1u);
+  __syncthreads();
+  const uint32_t lt = (uint32_t)uniform_i((int)long_ticket);
+  if (lt < nlong) {
+    if (half == 1) return;
+    geo_long::GeoWave gl;
+    gl.lane = lane;
+    gl.L = &reinterpret_cast<geo_long::GeoShared*>(lds)->a;
+    gl.ws = slot;
+    gl.heapSize = 0;
+    gl.nodeCount = 0;
+    gl.linkSpills = gl.heapSpills = 0;
+    int cls = 0;
+    while (lt >= first[cls + 1]) cls++;
+    const GeoQuery q = queries[(size_t)cls * stride + (lt - first[cls])];
+    serve_query(gl, nav, q, cls, out, last_cost, T);
+    linkSpills += gl.linkSpills; heapSpills += gl.heapSpills;
+  }
+  geo::GeoWave g;
+  g.lane = lane;
+  g.L = &reinterpret_cast<geo::GeoShared*>(lds + (size_t)half * kHalf)->a;
+  g.ws = slot;
+  g.heapSize = 0;
+  g.nodeCount = 0;
+  g.linkSpills = g.heapSpills = 0;
+  // tickets below `taken` went to the blocks' first wavefronts above
+  const uint32_t taken = nlong < gridDim.x ? nlong : gridDim.x;
   for (;;) {
     uint32_t qi = 0;
-    if (g.lane == 0) qi = atomicAdd(head, 1u);
+    if (lane == 0) qi = atomicAdd(head, 1u);
     qi = (uint32_t)uniform_i((int)qi);
     if (qi >= nq) break;
+    if (qi < taken) continue;
     int cls = 0;
     while (qi >= first[cls + 1]) cls++;
     const GeoQuery q = queries[(size_t)cls * stride + (qi - first[cls])];
-    const uint32_t pops0 = pops;
-#ifdef BPSX_QUERY_TRACE
-    const unsigned long long trace_t0 = wall_clock64();
-    g.missTop = g.missNb = g.maxHeap = 0;
-    const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
-#endif
-    set_wave_priority((kGeoClasses - 1 - cls) >> 2);   // the longer the expected search, the sooner its instructions issue
-#ifdef BPSX_PHASE_TIMING
-    const float d = geodesic_query(g, nav, q, &pops, &corridor, phase_acc);
-#else
-    const float d = geodesic_query(g, nav, q, &pops, &corridor);
-#endif
-    if (g.lane == 0) {
-#ifdef BPSX_QUERY_TRACE
-      const unsigned int ti = atomicAdd(&g_trace_n, 1u);
-      if (ti < (1u << 17)) {
-        g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = pops - pops0;
-        g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)(g.missTop & 0xfffu) << 24) |
-                          ((unsigned long long)(g.missNb & 0xfffu) << 36) | ((unsigned long long)(g.maxHeap & 0xffu) << 48);
-      }
-#endif
-      out[q.out] = d;
-      // estimate for the agent's next search: this one's length, decaying from earlier peaks
-      if (last_cost && q.cost_slot != kNoCostSlot) {
-        const uint32_t prev = last_cost[q.cost_slot], now = pops - pops0;
-        const uint32_t faded = prev == kCostUnknown ? 0u : prev - (prev >> 2);
-        last_cost[q.cost_slot] = now > faded ? now : faded;
-      }
-    }
-    done++;
-    wave_sync();
+    serve_query(g, nav, q, cls, out, last_cost, T);
   }
-  if (g.lane == 0 && done) {
-    atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)done);
-    atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)pops);
-    atomicAdd((unsigned long long*)&counters[kCntCorridor], (unsigned long long)corridor);
-    if (g.linkSpills) atomicAdd((unsigned long long*)&counters[kCntLinkSpills], (unsigned long long)g.linkSpills);
-    if (g.heapSpills) atomicAdd((unsigned long long*)&counters[kCntHeapSpills], (unsigned long long)g.heapSpills);
+  linkSpills += g.linkSpills; heapSpills += g.heapSpills;
+  if (lane == 0 && T.done) {
+    atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)T.done);
+    atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)T.pops);
+    atomicAdd((unsigned long long*)&counters[kCntCorridor], (unsigned long long)T.corridor);
+    if (linkSpills) atomicAdd((unsigned long long*)&counters[kCntLinkSpills], (unsigned long long)linkSpills);
+    if (heapSpills) atomicAdd((unsigned long long*)&counters[kCntHeapSpills], (unsigned long long)heapSpills);
 #ifdef BPSX_PHASE_TIMING
-    for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], phase_acc[k]);
+    for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], T.phase_acc[k]);
 #endif
   }
 }
@@ -540,8 +604,9 @@ __global__ void k_random_points(NavData nav, uint32_t scene, const float* u, uin
   oxyz[(size_t)i * 3] = p[0]; oxyz[(size_t)i * 3 + 1] = p[1]; oxyz[(size_t)i * 3 + 2] = p[2];
   oref[i] = ok ? (s.ref_base | ip) : 0;
 }
+// counts and both ticket counters of a batch of n queries, all in the class of the shortest
 __global__ void k_set_counts(uint32_t* p, uint32_t n) {
-  if (threadIdx.x <= (uint32_t)kGeoClasses) p[threadIdx.x] = threadIdx.x == 0 ? n : 0u;
+  if (threadIdx.x <= (uint32_t)kGeoClasses + 1u) p[threadIdx.x] = threadIdx.x == (uint32_t)kGeoClasses - 1u ? n : 0u;
 }
 
 }  // namespace
@@ -551,15 +616,16 @@ static inline dim3 grid_for(uint32_t n, uint32_t block) { return dim3((n + block
 
 uint32_t geodesic_blocks_per_cu() {
   int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_geodesic, 64, 0) != hipSuccess || n < 1) n = 1;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, k_geodesic, 128, 0) != hipSuccess || n < 1) n = 1;
   return (uint32_t)n;
 }
 
+// num_blocks blocks of two wavefronts; slots holds one GeoSlot per wavefront
 void launch_geodesic(const NavData& nav, const GeoQuery* queries, uint32_t stride, const uint32_t* counts, uint32_t* head,
-                     float* out, uint32_t* last_cost, GeoSlot* slots, uint32_t num_blocks, uint64_t* counters,
-                     hipStream_t st) {
-  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(64), 0, st, nav, queries, stride, counts, head, out, last_cost,
-                     slots, counters);
+                     uint32_t* head_long, float* out, uint32_t* last_cost, GeoSlot* slots, uint32_t num_blocks,
+                     uint64_t* counters, hipStream_t st) {
+  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(128), 0, st, nav, queries, stride, counts, head, head_long, out,
+                     last_cost, slots, counters);
 }
 
 void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
@@ -573,8 +639,8 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   mark();
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, P);
   mark();
-  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, A.last_cost, slots, geo_blocks,
-                  P.counters, st);
+  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
+                  A.last_cost, slots, geo_blocks, P.counters, st);
   mark();
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
   mark();
@@ -585,8 +651,8 @@ void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q,
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
   hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, P);
-  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo, A.last_cost, slots, geo_blocks,
-                  P.counters, st);
+  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
+                  A.last_cost, slots, geo_blocks, P.counters, st);
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
 }
 
@@ -599,12 +665,13 @@ void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz
   hipLaunchKernelGGL(k_try_step_batch, grid_for(n, 64), dim3(64), 0, st, nav, scene, sxyz, sref, exyz, n, oxyz, oref);
 }
 void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
-                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 1] */, float* out,
+                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 2] */, float* out,
                            GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st) {
   hipLaunchKernelGGL(k_make_queries, grid_for(n, 256), dim3(256), 0, st, scene, sxyz, sref, exyz, eref, n, qbuf);
-  // all in the first class
   hipLaunchKernelGGL(k_set_counts, dim3(1), dim3(64), 0, st, count_head, n);
-  launch_geodesic(nav, qbuf, n, &count_head[0], &count_head[kGeoClasses], out, nullptr, slots, geo_blocks, counters, st);
+  // one class only: stride 0 puts its queries at the start of the buffer
+  launch_geodesic(nav, qbuf, 0, &count_head[0], &count_head[kGeoClasses], &count_head[kGeoClasses + 1], out, nullptr, slots,
+                  geo_blocks, counters, st);
 }
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,
                           hipStream_t st) {
