@@ -527,6 +527,7 @@ __global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* _
     const GeoQuery q = queries[(size_t)cls * stride + (lt - first[cls])];
     serve_query(gl, nav, q, cls, out, last_cost, T);
     linkSpills += gl.linkSpills; heapSpills += gl.heapSpills;
+    if (lane == 0) atomicAdd((unsigned long long*)&counters[kCntLongPath], 1ull);
   }
   geo::GeoWave g;
   g.lane = lane;

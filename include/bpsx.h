@@ -150,8 +150,10 @@ int bpsx_check_errors(bpsx_sim *sim);
  * [7] snap candidates; [8..15] are zero unless the library was built with -DBPSX_PHASE_TIMING
  * (cycle counts of the A* loop's phases, a diagnostic build); [16] path searches that needed
  * more node links than the kernel keeps in LDS, [17] path searches whose open list outgrew
- * the kernel's registers (both continue in slower code; results are the same). */
-#define BPSX_NUM_COUNTERS 18
+ * the kernel's registers (both continue in slower code; results are the same), [18] path
+ * searches expected to be among the longest of their step, which the kernel runs with larger
+ * LDS structures (same results). */
+#define BPSX_NUM_COUNTERS 19
 int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
 /* Per-kernel timing with HIP events on the step's own stream. While enabled, every
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the

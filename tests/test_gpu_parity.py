@@ -388,6 +388,9 @@ def test_full_size_workload_properties(oracle, torch_cuda):
         if rep == 0:
             cnt = gen.counters()
             assert cnt["agent_steps"] == N * steps and cnt["geodesic_queries"] > N
+            # the kernel's path for the searches expected to be longest, and its link-spill path
+            # for the others, both took part in what is compared with the oracle below
+            assert cnt["geo_long_path"] > 100 and cnt["geo_link_spills"] > 100
         gen.check_errors()
         gen.close()
     for k in runs[0]:
