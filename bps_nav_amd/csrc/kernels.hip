@@ -5,10 +5,11 @@
 //                  observation, and a geodesic query (goal -> agent) when the agent moved or
 //                  the episode ended; an agent whose episode ended also picks its next episode
 //                  here and is queued for reset (simulator.cpp:620-632, 651-710, 601-610)
-//   reset_snap     wavefront per queued agent: snap start and goal of the new episode, polar,
-//                  and the new episode's first query (agent -> goal)
+//   reset_snap     two wavefronts per queued agent: snap start and goal of the new episode,
+//                  polar, and the new episode's first query (agent -> goal)
 //                                                        (simulator.cpp:611-614, 744-751)
-//   geodesic       wavefront per query, both kinds in one launch: A* + funnel
+//   geodesic       wavefront per query, both kinds in one launch: A* + funnel; blocks of two
+//                  wavefronts so that the longest searches can take a block's whole LDS
 //                                                        (PathFinder.cpp:485-541)
 //   step_finish    lane per agent: info, reward, mask from the terminal transition, then the
 //                  new episode's distance bookkeeping    (simulator.cpp:634-641, 758-822, 749-755)
