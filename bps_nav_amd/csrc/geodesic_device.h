@@ -681,6 +681,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
   }
 #undef ASTAR_RUN
   (void)ex;
+  if (st.outOfNodes) return 0;   // no path to build: the result is a failure
   const int lastBest = st.lastBest;
   // getPathToNode: one walk up the parents notes the node indices (in the window's array of
   // positions, no longer needed), then all lanes fill the corridor, which overlays the hash heads;
