@@ -169,6 +169,7 @@ BPSX_DEV void begin_reset(const NavData& nav, const AgentArrays& A, const StepPa
 
 __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, StepQueues Q, StepParams P,
                                                    const int64_t* __restrict__ actions) {
+  __shared__ MoveLds move_lds;
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   bool want = false, reset = false;
   uint32_t cls = 0;
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
           NavPt st;
           st.x = A.nav_xyz[(size_t)gi * 3]; st.y = A.nav_xyz[(size_t)gi * 3 + 1]; st.z = A.nav_xyz[(size_t)gi * 3 + 2];
           st.ref = A.nav_ref[gi];
-          const NavPt r = try_step(nav, s, st, pos[0] + delta[0], pos[1] + delta[1], pos[2] + delta[2], &movePolys);
+          const NavPt r = try_step(nav, s, st, pos[0] + delta[0], pos[1] + delta[1], pos[2] + delta[2], &movePolys, move_lds);
           samePoint = __float_as_uint(r.x) == __float_as_uint(st.x) && __float_as_uint(r.y) == __float_as_uint(st.y) &&
                       __float_as_uint(r.z) == __float_as_uint(st.z) && r.ref == st.ref;
           pos[0] = r.x; pos[1] = r.y; pos[2] = r.z;
@@ -578,11 +579,12 @@ __global__ __launch_bounds__(64) void k_snap_batch(NavData nav, uint32_t scene, 
 }
 __global__ void k_try_step_batch(NavData nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
                                  uint32_t n, float* oxyz, uint32_t* oref) {
+  __shared__ MoveLds move_lds;
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   uint32_t c = 0;
   NavPt st{sxyz[(size_t)i * 3], sxyz[(size_t)i * 3 + 1], sxyz[(size_t)i * 3 + 2], sref[i]};
-  const NavPt r = try_step(nav, nav.scenes[scene], st, exyz[(size_t)i * 3], exyz[(size_t)i * 3 + 1], exyz[(size_t)i * 3 + 2], &c);
+  const NavPt r = try_step(nav, nav.scenes[scene], st, exyz[(size_t)i * 3], exyz[(size_t)i * 3 + 1], exyz[(size_t)i * 3 + 2], &c, move_lds);
   oxyz[(size_t)i * 3] = r.x; oxyz[(size_t)i * 3 + 1] = r.y; oxyz[(size_t)i * 3 + 2] = r.z;
   oref[i] = r.ref;
 }

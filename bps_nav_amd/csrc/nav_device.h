@@ -339,18 +339,26 @@ BPSX_DEV NavPt snap_point_wave(const NavData& nav, const SceneDev& s, float px, 
   return out;
 }
 
+// The tiny node pool and the queue of moveAlongSurface, one column per lane of a wavefront, in
+// LDS: they are indexed at run time, which in private memory means a trip to scratch (HBM
+// behind the vector caches) per access.  A node enters the queue at most once, so the queue
+// needs no more entries than there are nodes and is never shifted: `head` moves instead.
+struct MoveLds {
+  uint16_t node_id[kTinyNodes][64];
+  uint8_t queue[kTinyNodes][64];
+};
+
 // tryStep with sliding, one lane per agent.
 BPSX_DEV NavPt try_step(const NavData& nav, const SceneDev& s, const NavPt& start, float ex, float ey, float ez,
-                        uint32_t* npolys) {
+                        uint32_t* npolys, MoveLds& M) {
   const uint32_t startIp = decode_ref(s, start.ref);
   if (startIp == kInvalidPoly || !finite3(start.x, start.y, start.z) || !finite3(ex, ey, ez)) return start;
-  uint16_t nodeId[kTinyNodes];
+  const int lane = (int)(threadIdx.x & 63);
   uint64_t closed = 1ull;
   int nnodes = 1;
-  uint8_t queue[kMoveQueue];
-  int nqueue = 1;
-  nodeId[0] = (uint16_t)startIp;
-  queue[0] = 0;
+  int qhead = 0, qtail = 1;   // the reference's stack holds entries [qhead, qtail)
+  M.node_id[0][lane] = (uint16_t)startIp;
+  M.queue[0][lane] = 0;
   float bx = start.x, by = start.y, bz = start.z;
   float bestDist = 3.402823466e+38f;
   int bestNode = -1;
@@ -358,11 +366,9 @@ BPSX_DEV NavPt try_step(const NavData& nav, const SceneDev& s, const NavPt& star
   const float ddx = ex - start.x, ddy = ey - start.y, ddz = ez - start.z;
   const float sr = sqrtf(ddx * ddx + ddy * ddy + ddz * ddz) / 2.0f + 0.001f;
   const float searchRadSqr = sr * sr;
-  while (nqueue) {
-    const int cur = queue[0];
-    for (int i = 0; i < nqueue - 1; ++i) queue[i] = queue[i + 1];
-    nqueue--;
-    const PolyRec& r = nav.polys[s.poly_base + nodeId[cur]];
+  while (qhead < qtail) {
+    const int cur = M.queue[qhead++][lane];
+    const PolyRec& r = nav.polys[s.poly_base + M.node_id[cur][lane]];
     (*npolys)++;
     if (point_in_poly(ex, ez, r)) {
       bestNode = cur;
@@ -389,28 +395,29 @@ BPSX_DEV NavPt try_step(const NavData& nav, const SceneDev& s, const NavPt& star
         const uint16_t ip = (uint16_t)(nb - 1);
         int nn = -1;
         for (int k = 0; k < nnodes; ++k)
-          if (nodeId[k] == ip) { nn = k; break; }
+          if (M.node_id[k][lane] == ip) { nn = k; break; }
         if (nn < 0) {
           if (nnodes >= kTinyNodes) continue;
           nn = nnodes++;
-          nodeId[nn] = ip;
+          M.node_id[nn][lane] = ip;
         }
         if ((closed >> nn) & 1ull) continue;
         float t;
         const float d = dist_pt_seg_sqr2d(sx, sz, vj, vi, t);
         if (d > searchRadSqr) continue;
-        if (nqueue < kMoveQueue) {
+        if (qtail - qhead < kMoveQueue) {
           closed |= 1ull << nn;
-          queue[nqueue++] = (uint8_t)nn;
+          M.queue[qtail++][lane] = (uint8_t)nn;
         }
       }
     }
   }
   if (bestNode < 0) return start;
-  NavPt out{bx, by, bz, s.ref_base | (uint32_t)nodeId[bestNode]};
+  const uint32_t bestIp = M.node_id[bestNode][lane];
+  NavPt out{bx, by, bz, s.ref_base | bestIp};
   if (isfinite(bx) && isfinite(bz)) {
     float h;
-    if (poly_height(nav, nav.polys[s.poly_base + nodeId[bestNode]], bx, by, bz, h)) out.y = h;
+    if (poly_height(nav, nav.polys[s.poly_base + bestIp], bx, by, bz, h)) out.y = h;
   }
   return out;
 }
