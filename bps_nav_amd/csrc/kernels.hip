@@ -264,7 +264,24 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
       }
     }
   }
-  if (want) Q.queries[(size_t)cls * Q.stride + atomicAdd(&Q.counts[kQGeo + cls], 1u)] = q;
+  // queue the queries: one atomic per wavefront and class present in it (per-lane atomics on
+  // the sixteen class counters serialise)
+  {
+    const int lane = (int)(threadIdx.x & 63);
+    uint32_t slot = 0;
+    unsigned long long todo = __ballot(want);
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const uint32_t c = (uint32_t)__shfl((int)cls, leader);
+      const unsigned long long same = __ballot(want && cls == c);
+      uint32_t base = 0;
+      if (lane == leader) base = atomicAdd(&Q.counts[kQGeo + c], (uint32_t)__popcll(same));
+      base = (uint32_t)__shfl((int)base, leader);
+      if (want && cls == c) slot = base + (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
+      todo &= ~same;
+    }
+    if (want) Q.queries[(size_t)cls * Q.stride + slot] = q;
+  }
   const uint32_t rslot = wave_append(reset, &Q.counts[kQReset]);
   if (reset) Q.reset_list[rslot] = gi;
   // counters, one atomic per wavefront
