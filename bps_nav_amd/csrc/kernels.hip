@@ -183,7 +183,20 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
       atomicOr(P.error_flag, 1u);
       A.flags[gi] = kAgentSkip;
     } else {
+      // Everything the step may need of the agent is read here, before the first store: the
+      // loads then go out together instead of one dependent round trip after the other.
       const uint32_t step = A.step[gi] + 1;
+      const uint32_t scene0 = A.scene[gi];
+      float pos[3], rot[4], goal[3], navNow[3], goalNav[3];
+      load3(A.pos, gi, pos);
+      load3(A.goal, gi, goal);
+      for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
+      load3(A.nav_xyz, gi, navNow);
+      uint32_t navRefNow = A.nav_ref[gi];
+      load3(A.goal_xyz, gi, goalNav);
+      const uint32_t goalRef = A.goal_ref[gi];
+      const bool distOk = A.dist_ok[gi] != 0;
+      const uint32_t expected = A.last_cost[gi];
       A.step[gi] = step;
       bool done = (float)step >= P.max_steps;
       bool moved = false;
@@ -194,22 +207,18 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
       if (action == 0) {
         done = true;
       } else {
-        float pos[3], rot[4], goal[3];
-        load3(A.pos, gi, pos);
-        load3(A.goal, gi, goal);
-        for (int k = 0; k < 4; ++k) rot[k] = A.rot[(size_t)gi * 4 + k];
         if (action == 1) {
           const float fwd[3] = {0.f * 0.25f, 0.f * 0.25f, -1.f * 0.25f};
           float delta[3];
           quat_rotate(rot, fwd, delta);
-          const SceneDev& s = nav.scenes[A.scene[gi]];
-          NavPt st;
-          st.x = A.nav_xyz[(size_t)gi * 3]; st.y = A.nav_xyz[(size_t)gi * 3 + 1]; st.z = A.nav_xyz[(size_t)gi * 3 + 2];
-          st.ref = A.nav_ref[gi];
+          const SceneDev& s = nav.scenes[scene0];
+          const NavPt st{navNow[0], navNow[1], navNow[2], navRefNow};
           const NavPt r = try_step(nav, s, st, pos[0] + delta[0], pos[1] + delta[1], pos[2] + delta[2], &movePolys, move_lds);
           samePoint = __float_as_uint(r.x) == __float_as_uint(st.x) && __float_as_uint(r.y) == __float_as_uint(st.y) &&
                       __float_as_uint(r.z) == __float_as_uint(st.z) && r.ref == st.ref;
           pos[0] = r.x; pos[1] = r.y; pos[2] = r.z;
+          navNow[0] = r.x; navNow[1] = r.y; navNow[2] = r.z;
+          navRefNow = r.ref;
           store3(A.nav_xyz, gi, pos);
           A.nav_ref[gi] = r.ref;
           store3(A.pos, gi, pos);
@@ -223,29 +232,23 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
       // PointNav measures the distance on every move and at the end of the episode, Flee on
       // moves only, Exploration never (simulator.cpp:758-790, 845-856, 918-927)
       const bool measure = P.task == BPSX_TASK_POINTNAV ? (done || moved) : (P.task == BPSX_TASK_FLEE && moved);
-      const bool reuse = measure && samePoint && A.dist_ok[gi] != 0;
+      const bool reuse = measure && samePoint && distOk;
       A.flags[gi] = (done ? kAgentDone : 0u) | (moved ? kAgentMoved : 0u) | (reuse ? kAgentReuse : 0u);
       if (P.task == BPSX_TASK_EXPLORATION) {
         // the count is taken before the pose arrays move on to the next episode
         uint32_t cnt = A.exp_count[gi];
-        if (moved) {
-          float pos[3];
-          load3(A.pos, gi, pos);
-          cnt = visit_cell(A, gi, pos);
-        }
+        if (moved) cnt = visit_cell(A, gi, pos);
         A.geo[gi] = (float)(cnt - 1);
       }
       if (measure && !reuse) {
         want = true;
-        load3(A.goal_xyz, gi, q.a);
-        q.a_ref = A.goal_ref[gi];
-        load3(A.nav_xyz, gi, q.b);
-        q.b_ref = A.nav_ref[gi];
-        q.scene = A.scene[gi];
+        for (int k = 0; k < 3; ++k) { q.a[k] = goalNav[k]; q.b[k] = navNow[k]; }
+        q.a_ref = goalRef;
+        q.b_ref = navRefNow;
+        q.scene = scene0;
         q.out = gi;
         q.cost_slot = done ? kNoCostSlot : gi;   // a finished episode's search predicts nothing
         q.pad = 0;
-        const uint32_t expected = A.last_cost[gi];
         cls = expected == kCostUnknown ? kGeoClassUnknown : geo_class(expected);
       }
       if (done) {
@@ -253,7 +256,7 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
         // take the next episode now; distance bookkeeping waits for step_finish.  If a new scene
         // waits for this env's slot, the next episode is drawn there (simulator.cpp:1636-1642).
         {
-          const uint32_t cur = A.scene[gi], tgt = P.swap_target[cur % P.num_slots];
+          const uint32_t cur = scene0, tgt = P.swap_target[cur % P.num_slots];
           if (tgt != kNoSwap && tgt != cur) {
             A.scene[gi] = tgt;
             atomicSub(&P.swap_remaining[cur % P.num_slots], 1u);
@@ -264,23 +267,21 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
       }
     }
   }
-  // queue the queries: one atomic per wavefront and class present in it (per-lane atomics on
-  // the sixteen class counters serialise)
+  // queue the queries: one atomic per wavefront and class present in it, all of them in flight
+  // together (per-lane atomics on the sixteen class counters serialise, and so do the round
+  // trips of one atomic per class after the other)
   {
     const int lane = (int)(threadIdx.x & 63);
-    uint32_t slot = 0;
-    unsigned long long todo = __ballot(want);
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const uint32_t c = (uint32_t)__shfl((int)cls, leader);
-      const unsigned long long same = __ballot(want && cls == c);
-      uint32_t base = 0;
-      if (lane == leader) base = atomicAdd(&Q.counts[kQGeo + c], (uint32_t)__popcll(same));
-      base = (uint32_t)__shfl((int)base, leader);
-      if (want && cls == c) slot = base + (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
-      todo &= ~same;
+    unsigned long long mine = 0;   // lanes of this wavefront that queue into the same class as this one
+    for (uint32_t c = 0; c < (uint32_t)kGeoClasses; ++c) {
+      const unsigned long long m = __ballot(want && cls == c);
+      if (want && cls == c) mine = m;
     }
-    if (want) Q.queries[(size_t)cls * Q.stride + slot] = q;
+    const int leader = want ? __ffsll((long long)mine) - 1 : lane;
+    uint32_t base = 0;
+    if (want && lane == leader) base = atomicAdd(&Q.counts[kQGeo + cls], (uint32_t)__popcll(mine));
+    base = (uint32_t)__shfl((int)base, leader);
+    if (want) Q.queries[(size_t)cls * Q.stride + base + (uint32_t)__popcll(mine & ((1ull << lane) - 1ull))] = q;
   }
   const uint32_t rslot = wave_append(reset, &Q.counts[kQReset]);
   if (reset) Q.reset_list[rslot] = gi;
