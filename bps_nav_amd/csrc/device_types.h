@@ -176,7 +176,7 @@ constexpr uint32_t kCostUnknown = 0xffffffffu;
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,
-  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18   // 8..15: phase cycles of the diagnostic build
+  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18, kCntTieRestarts = 19   // 8..15: phase cycles of the diagnostic build
 };
 
 }  // namespace bpsx

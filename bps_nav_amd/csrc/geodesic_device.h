@@ -36,6 +36,9 @@
 
 #ifndef BPSX_GEODESIC_COMMON_H
 #define BPSX_GEODESIC_COMMON_H
+#ifndef BPSX_BAG
+#define BPSX_BAG 0   // 1: searches start with the open list as an unordered set (see OpenBag)
+#endif
 namespace bpsx {
 
 #ifdef BPSX_ASM_MARKS
@@ -217,13 +220,99 @@ struct RegHeap {
   }
 };
 
+// The open list as an unordered set in registers.  dtNodeQueue::pop returns the entry with the
+// smallest total; while that smallest total is held by one entry only, which entry that is does
+// not depend on how the binary heap happens to be arranged, so a set with a minimum search gives
+// the same sequence of pops as the heap.  Entry p (0-based, dense: entries 0..size-1) lives in
+// lane p & 63 of register pair p >> 6.  The minimum is found with a cross-lane reduction; push
+// appends, modify rewrites the key of the entry that names the node, pop moves the last entry
+// into the gap.  When two entries share the smallest total the heap's arrangement decides, and
+// the search is run again with the exact heap (RegHeap).
+struct OpenBag {
+  static constexpr int kRegs = 4;
+  static constexpr int kCap = 64 * kRegs;
+  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
+  uint32_t t[kRegs];   // total bits
+  uint32_t n[kRegs];   // node index (bits 0-10) | the node's polygon index << 11
+  int size;
+  BPSX_DEV void init() {
+#pragma unroll
+    for (int r = 0; r < kRegs; ++r) { t[r] = kEmpty; n[r] = 0; }
+    size = 0;
+  }
+  static BPSX_DEV uint32_t dpp_min(uint32_t v, uint32_t w) { return w < v ? w : v; }
+  // smallest key of the wavefront, the same value in every lane's return
+  static BPSX_DEV uint32_t wave_min(uint32_t v) {
+    // within rows of 16 lanes: butterfly over 1, 2, then mirror within 8, mirror within 16
+    v = dpp_min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, false));
+    v = dpp_min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, false));
+    v = dpp_min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x141 /* row_half_mirror */, 0xf, 0xf, false));
+    v = dpp_min(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x140 /* row_mirror */, 0xf, 0xf, false));
+    // every lane now holds its row's minimum: combine the four rows on the scalar unit
+    const uint32_t a = rlane(v, 0), b = rlane(v, 16), c = rlane(v, 32), d = rlane(v, 48);
+    const uint32_t ab = a < b ? a : b, cd = c < d ? c : d;
+    return ab < cd ? ab : cd;
+  }
+  BPSX_DEV uint32_t key_at(int p) const {
+    const int l = p & 63;
+    switch (p >> 6) { case 0: return rlane(t[0], l); case 1: return rlane(t[1], l); case 2: return rlane(t[2], l); default: return rlane(t[3], l); }
+  }
+  BPSX_DEV uint32_t node_at(int p) const {
+    const int l = p & 63;
+    switch (p >> 6) { case 0: return rlane(n[0], l); case 1: return rlane(n[1], l); case 2: return rlane(n[2], l); default: return rlane(n[3], l); }
+  }
+  BPSX_DEV void set(int p, uint32_t key, uint32_t node) {
+    const int l = p & 63;
+    switch (p >> 6) {
+      case 0: t[0] = wlane(t[0], key, l); n[0] = wlane(n[0], node, l); break;
+      case 1: t[1] = wlane(t[1], key, l); n[1] = wlane(n[1], node, l); break;
+      case 2: t[2] = wlane(t[2], key, l); n[2] = wlane(n[2], node, l); break;
+      default: t[3] = wlane(t[3], key, l); n[3] = wlane(n[3], node, l); break;
+    }
+  }
+  // Position of the entry with the smallest total; *tie when another entry has the same total.
+  BPSX_DEV int argmin(bool* tie) const {
+    uint32_t m01 = t[0] < t[1] ? t[0] : t[1], m23 = t[2] < t[3] ? t[2] : t[3];
+    if (size <= 128) m23 = kEmpty;
+    const uint32_t m = wave_min(m01 < m23 ? m01 : m23);
+    const unsigned long long h0 = __ballot(t[0] == m), h1 = __ballot(t[1] == m);
+    int count = __popcll(h0) + __popcll(h1);
+    int pos = h0 ? __ffsll((long long)h0) - 1 : 64 + __ffsll((long long)h1) - 1;
+    if (size > 128) {
+      const unsigned long long h2 = __ballot(t[2] == m), h3 = __ballot(t[3] == m);
+      count += __popcll(h2) + __popcll(h3);
+      if (!(h0 | h1)) pos = h2 ? 128 + __ffsll((long long)h2) - 1 : 192 + __ffsll((long long)h3) - 1;
+    }
+    *tie = count > 1;
+    return pos;
+  }
+  // takes entry p out: the last entry moves into its place
+  BPSX_DEV void remove(int p) {
+    const int last = size - 1;
+    size = last;
+    const uint32_t lt = key_at(last), ln = node_at(last);
+    set(last, kEmpty, 0);
+    if (p != last) set(p, lt, ln);
+  }
+  BPSX_DEV void push(uint32_t key, uint32_t node) {
+    set(size, key, node);
+    size++;
+  }
+  // the entry of node `node` (packed like n[]) gets key `key`
+  BPSX_DEV void modify(uint32_t node, uint32_t key) {
+#pragma unroll
+    for (int r = 0; r < kRegs; ++r) t[r] = (n[r] == node && t[r] != kEmpty) ? key : t[r];
+  }
+};
+
 struct AstarState {
   int lastBest;
   float lastBestCost;
   bool outOfNodes;
   RegHeap rh;
+  OpenBag bag;
 };
-enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
+enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3, kAstarTie = 4 };
 
 BPSX_DEV float tri_area2d(const float* a, const float* b, const float* c) {
   const float abx = b[0] - a[0], abz = b[2] - a[2];
@@ -298,6 +387,7 @@ struct GeoWave {
   int heapSize;
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
+  uint32_t tieRestarts;              // queries run again with the exact heap
 #ifdef BPSX_QUERY_TRACE
   uint32_t missTop, missNb, maxHeap;
 #endif
@@ -419,9 +509,12 @@ struct GeoWave {
   }
 };
 
-// The expansion loop of findPath.  M = 0: open list in registers, all links in LDS; M = 1: open
-// list in registers, links may spill; M = 2: open list in LDS/HBM, links may spill.  Returns
-// kAstarGrow* before an expansion that could outgrow what its mode holds.
+// The expansion loop of findPath.  M = 3: open list as an unordered set in registers, all links
+// in LDS; M = 4: the same, links may spill.  These two return kAstarTie when two open entries
+// share the smallest total; the search then starts again with the exact heap: M = 0: heap in
+// registers, all links in LDS; M = 1: heap in registers, links may spill; M = 2: heap in
+// LDS/HBM, links may spill.  Returns kAstarGrow* before an expansion that could outgrow what
+// its mode holds.
 template <int M>
 BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
 #ifdef BPSX_PHASE_TIMING
@@ -433,17 +526,30 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const float H_SCALE = 0.999f;
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
   endIp = (uint32_t)uniform_i((int)endIp);   // the same in all lanes: the goal test stays on the scalar unit
-  constexpr bool S = M >= 1;    // links and states may be in HBM
+  constexpr bool S = M == 1 || M == 2 || M == 4;    // links and states may be in HBM
   constexpr bool SH = M == 2;   // open list in LDS/HBM
+  constexpr bool BAG = M >= 3;  // open list as an unordered set
   RegHeap& rh = st.rh;
-  while ((SH ? g.heapSize : rh.size) > 0) {
-    if (M == 0 && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
-    if (!SH && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
-    // the node about to be popped is the root: fetch its edges while the heap is repaired
+  OpenBag& bag = st.bag;
+  while ((SH ? g.heapSize : (BAG ? bag.size : rh.size)) > 0) {
+    if (!S && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
+    if (!SH && !BAG && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
+    if (BAG && bag.size > OpenBag::kCap - kNvp) return kAstarGrowHeap;
+    // the node about to be popped is known before the open list is repaired: fetch its edges
+    // meanwhile
     int bi;
     uint32_t bestIp;
     uint32_t blink;   // the node's link word: closing the node rewrites its flags
-    if (SH) {
+    int bagPos = 0;
+    if (BAG) {
+      bool tie;
+      bagPos = bag.argmin(&tie);
+      if (tie) return kAstarTie;
+      const uint32_t root = bag.node_at(bagPos);
+      bi = (int)(root & 0x7ffu);
+      bestIp = root >> 11;
+      blink = g.link<S>(bi);
+    } else if (SH) {
       bi = uniform_i((int)L->heap[0].node);
       blink = g.link<S>(bi);
       bestIp = link_id((uint32_t)uniform_i((int)blink));
@@ -480,7 +586,8 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (!SH && (uint32_t)rh.size > g.maxHeap) g.maxHeap = (uint32_t)rh.size;
 #endif
     PHASE_MARK(0);
-    if (SH) g.pop<true>();
+    if (BAG) bag.remove(bagPos);
+    else if (SH) g.pop<true>();
     else rh.pop(lane);
     const uint32_t pidx = (uint32_t)uniform_i((int)bparent);
     PHASE_MARK(1);
@@ -602,7 +709,10 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const uint32_t entry = rlane(packed, src);
       const float t = lane_f(total, src);
       const bool open = (openMask >> src) & 1ull;
-      if (SH) {
+      if (BAG) {
+        if (open) bag.modify(entry, __float_as_uint(t));
+        else bag.push(__float_as_uint(t), entry);
+      } else if (SH) {
         if (open) g.modify<true>((int)(entry & 0x7ffu), t);
         else g.push<true>(t, (int)(entry & 0x7ffu));
       } else {
@@ -639,8 +749,9 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #else
 #define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
 #endif
-  g.clear();
-  {
+  float startTotal;
+  auto begin = [&]() {
+    g.clear();
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
     const float total = sqrtf(dx * dx + dy * dy + dz * dz) * 0.999f;
     g.nodeCount = 1;
@@ -659,11 +770,26 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.lastBest = 0;
     st.lastBestCost = total;
     st.outOfNodes = false;
+    startTotal = total;
+  };
+  AstarExit ex = kAstarTie;
+#if BPSX_BAG
+  begin();
+  st.bag.init();
+  st.bag.push(__float_as_uint(startTotal), startIp << 11);
+  ex = ASTAR_RUN(3);
+  if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(4); }
+#endif
+  if (ex == kAstarTie || ex == kAstarGrowHeap) {
+    // two open entries shared the smallest total (or the set is full): the order of pops now
+    // depends on the heap's arrangement, so the search is done again with the heap itself
+    if (BPSX_BAG) g.tieRestarts++;
+    begin();
     st.rh.init();
-    st.rh.push(__float_as_uint(total), startIp << 11, lane);
+    st.rh.push(__float_as_uint(startTotal), startIp << 11, lane);
+    ex = ASTAR_RUN(0);
+    if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
   }
-  AstarExit ex = ASTAR_RUN(0);
-  if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
   if (ex == kAstarGrowHeap) {
     g.heapSpills++;
     // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap

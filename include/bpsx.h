@@ -152,8 +152,10 @@ int bpsx_check_errors(bpsx_sim *sim);
  * more node links than the kernel keeps in LDS, [17] path searches whose open list outgrew
  * the kernel's registers (both continue in slower code; results are the same), [18] path
  * searches expected to be among the longest of their step, which the kernel runs with larger
- * LDS structures (same results). */
-#define BPSX_NUM_COUNTERS 19
+ * LDS structures (same results), [19] path searches that met two open nodes with the same
+ * smallest total and were run again with the reference's binary heap, whose arrangement
+ * decides between them (same results). */
+#define BPSX_NUM_COUNTERS 20
 int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
 /* Per-kernel timing with HIP events on the step's own stream. While enabled, every
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
