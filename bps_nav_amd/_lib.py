@@ -92,6 +92,8 @@ def lib():
                                          C.c_uint32, C.c_void_p, C.c_void_p]
             L.bpsx_geodesic.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
                                         C.c_void_p, C.c_uint32, C.c_void_p]
+            L.bpsx_geodesic_static.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
+                                               C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p]
             L.bpsx_random_points.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib

@@ -273,6 +273,22 @@ class PointNavRolloutGenerator:
                                          eref.ctypes.data, n, out.ctypes.data))
         return out
 
+    STATIC_MAX_QUERIES = 4096     # BPSX_STATIC_MAX_QUERIES
+
+    def geodesic_static(self, scene, sxyz, sref, exyz, eref, out=None):
+        """bpsx_geodesic_static: device tensors in (f32[n,3], i32/u32 bit patterns [n]) and out
+        (f32[n]); enqueued on the current stream, no allocation inside the library."""
+        n = sxyz.shape[0]
+        for t_, dt in ((sxyz, torch.float32), (exyz, torch.float32), (sref, torch.int32), (eref, torch.int32)):
+            if not (t_.is_cuda and t_.is_contiguous() and t_.dtype == dt):
+                raise ValueError("geodesic_static takes contiguous device tensors: f32 points, int32 refs")
+        if out is None:
+            out = torch.empty(n, dtype=torch.float32, device=sxyz.device)
+        _lib.check(self._L.bpsx_geodesic_static(self._h, scene, C.c_void_p(sxyz.data_ptr()), C.c_void_p(sref.data_ptr()),
+                                                C.c_void_p(exyz.data_ptr()), C.c_void_p(eref.data_ptr()), n,
+                                                C.c_void_p(out.data_ptr()), self._stream()))
+        return out
+
     def random_points(self, scene, u):
         u = np.ascontiguousarray(u, np.float32).reshape(-1, 3)
         n = len(u)

@@ -4,6 +4,7 @@
 // kernels on the caller's HIP stream.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -45,6 +46,33 @@ int dev_alloc(T** p, size_t count) {
 }
 
 }  // namespace
+
+// ---- scratch of the allocation-free geodesic entry point (bpsx_geodesic_static).  One array per
+// GPU, held until the process ends: the queries built from the caller's arrays, the queue
+// counters, and the node pools of the kStaticBlocks * 2 wavefronts that serve the queue.
+namespace {
+constexpr uint32_t kStaticBlocks = 32;
+constexpr size_t kStaticQueriesBytes = (size_t)BPSX_STATIC_MAX_QUERIES * sizeof(GeoQuery);
+constexpr size_t kStaticCountsBytes = 256;
+static_assert((kGeoClasses + 2) * sizeof(uint32_t) <= kStaticCountsBytes, "queue counters must fit their part");
+static_assert(kStaticQueriesBytes % 256 == 0 && sizeof(GeoSlot) % 256 == 0, "parts of the scratch stay aligned");
+constexpr size_t kStaticSlotsBytes = (size_t)kStaticBlocks * 2 * sizeof(GeoSlot);
+constexpr size_t kStaticBytes = kStaticQueriesBytes + kStaticCountsBytes + kStaticSlotsBytes;
+constexpr int kMaxDevices = 64;
+unsigned char* g_static_scratch[kMaxDevices] = {};   // device address of `scratch` on each GPU that has been set up
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+// Looks the array's address up on the current device, once per device.
+static int static_scratch_setup(int device) {
+  if (device < 0 || device >= kMaxDevices) return fail(BPSX_E_UNSUPPORTED, "device ordinal beyond the table of static scratch arrays");
+  if (g_static_scratch[device]) return BPSX_OK;
+  unsigned char* ptr = nullptr;
+  HIP_TRY(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) return fail(BPSX_E_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+  g_static_scratch[device] = ptr;
+  return BPSX_OK;
+}
 
 // First-fit allocator over one of the concatenated navmesh arrays (units = elements).  Scenes
 // come and go with scene rotation; neighbouring free ranges are merged on release.
@@ -340,6 +368,9 @@ int bpsx_finalize(bpsx_sim* sim) {
     HIP_TRY(hipEventCreateWithFlags(&g.done, hipEventDisableTiming));
     for (auto& e : g.ev) HIP_TRY(hipEventCreate(&e));
   }
+  // the allocation-free entry point's scratch: its address on this device, looked up here so
+  // that the entry point itself makes no set-up call
+  if ((rc = static_scratch_setup(sim->cfg.gpu_id))) return rc;
   sim->finalized = true;
   return BPSX_OK;
 }
@@ -643,6 +674,28 @@ int bpsx_geodesic(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const u
                         sim->geo_blocks, sim->d_counters, nullptr);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipMemcpy(out_dist, d_o, u1, hipMemcpyDeviceToHost));
+  return BPSX_OK;
+}
+
+int bpsx_geodesic_static(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const uint32_t* start_ref,
+                         const float* end_xyz, const uint32_t* end_ref, uint32_t n, float* out_dist, void* hip_stream) {
+  int rc = check_scene(sim, scene, "geodesic_static");
+  if (rc) return rc;
+  if (n > BPSX_STATIC_MAX_QUERIES)
+    return fail(BPSX_E_INVAL, "geodesic_static: n = " + std::to_string(n) + " exceeds BPSX_STATIC_MAX_QUERIES = " +
+                                  std::to_string(BPSX_STATIC_MAX_QUERIES));
+  if (!n) return BPSX_OK;
+  if (!start_xyz || !start_ref || !end_xyz || !end_ref || !out_dist) return fail(BPSX_E_INVAL, "geodesic_static: null argument");
+  unsigned char* base = g_static_scratch[sim->cfg.gpu_id];   // set up by bpsx_finalize on this device
+  if (!base) return fail(BPSX_E_STATE, "geodesic_static: the static scratch array was not set up on this device");
+  GeoQuery* d_q = (GeoQuery*)base;
+  uint32_t* d_counts = (uint32_t*)(base + kStaticQueriesBytes);
+  GeoSlot* d_slots = (GeoSlot*)(base + kStaticQueriesBytes + kStaticCountsBytes);
+  // The counters are rewritten by a kernel at the start of every call; node pools and queries
+  // are written before they are read.  Nothing else of the previous call's contents is used.
+  launch_geodesic_batch(sim->nav, scene_entry(sim, scene), start_xyz, start_ref, end_xyz, end_ref, n, d_q, d_counts, out_dist,
+                        d_slots, std::min(kStaticBlocks, std::max(1u, (n + 1) / 2)), sim->d_counters, (hipStream_t)hip_stream);
+  HIP_TRY(hipGetLastError());
   return BPSX_OK;
 }
 

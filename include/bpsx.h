@@ -182,6 +182,19 @@ int bpsx_try_steps(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
 int bpsx_geodesic(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
                   const uint32_t *start_ref, const float *end_xyz, const uint32_t *end_ref,
                   uint32_t n, float *out_dist);
+/* bpsx_geodesic for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same distances as
+ * bpsx_geodesic, but every pointer is a DEVICE pointer, the work is enqueued on hip_stream and
+ * the call returns without waiting (out_dist is complete when the stream reaches that point),
+ * and the call allocates nothing: its queue and A* node pools live in an array of about 5.4 MB
+ * that each GPU the library runs on holds from library load until the process ends.  At most
+ * BPSX_STATIC_MAX_QUERIES queries per call (BPSX_E_INVAL beyond).  All calls on one GPU share
+ * that array: calls that overlap on one GPU (other streams, other simulators) race; calls on
+ * one stream are safe.  Must not be called between step_start and step_end. */
+#define BPSX_STATIC_MAX_QUERIES 4096
+int bpsx_geodesic_static(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
+                         const uint32_t *start_ref, const float *end_xyz, const uint32_t *end_ref,
+                         uint32_t n, float *out_dist, void *hip_stream);
 /* Area-weighted random navigable points (PathFinder.cpp:463-470; distribution of
  * dtNavMeshQuery::findRandomPoint, DetourNavMeshQuery.cpp:220-313).  u f32[n][3] are
  * uniform variates in [0,1): polygon pick, s, t. */
