@@ -23,13 +23,45 @@ HBM_PEAK_GBS = 8000.0
 # end polygons are read once more for the boundary clamp, 2 * (32 + 12 * nv) with nv = 4.
 BYTES_PER_CORRIDOR_POLY = 60
 BYTES_PER_QUERY_ENDS = 2 * (32 + 12 * 4)
-# HBM bytes per k_geodesic launch at the default workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this file (with --calib-copy), each scaled by what the counter reads for a 256 MiB copy.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 1.331e9
+# Counter figures of the dominant kernel (HBM bytes per launch, vector instructions per launch)
+# are not measured by this script: they come from rocprofv3 --pmc runs of this file whose
+# summary is tracked in profiles/.  That summary names the kernel sources it was measured on
+# (a hash); the figures are printed only while the sources are still the same, otherwise null.
+COUNTER_SUMMARY = os.path.join(ROOT, "profiles", "k_geodesic_c4_hbm_traffic.md")
+KERNEL_SOURCES = ("device_types.h", "kernels.h", "nav_device.h", "geodesic_device.h", "kernels.hip")
+# Vector-instruction issue peak: one wavefront instruction per cycle and SIMD of four-cycle
+# cadence, i.e. one per cycle and CU; 256 CUs at 2.4 GHz.
+VALU_ISSUE_PEAK = 256 * 2.4e9
 
 
 def log(*a):
     print("[bench]", *a, file=sys.stderr, flush=True)
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "bps_nav_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def tracked_counters():
+    """{name: value} from the `measured:` line of the tracked counter summary, or {} when the
+    summary is missing or was measured on other kernel sources."""
+    try:
+        with open(COUNTER_SUMMARY) as f:
+            lines = [ln for ln in f if ln.startswith("measured:")]
+    except OSError:
+        return {}
+    if not lines:
+        return {}
+    kv = dict(item.split("=", 1) for item in lines[-1].split()[1:])
+    if kv.get("kernel_source_sha16") != kernel_source_hash():
+        log(f"{os.path.relpath(COUNTER_SUMMARY, ROOT)} was measured on other kernel sources: counter figures not printed")
+        return {}
+    return kv
 
 
 def gpu_geodesic_fn(nav, scene):
@@ -58,22 +90,34 @@ def build_workload(num_scenes, episodes_per_scene):
     return out
 
 
-def cpu_baseline(workload, agents_per_scene, seed, p_forward, budget_s=20.0):
+def cpu_baseline(workload, agents_per_scene, seed, p_forward, budget_s=20.0, require_ref=False, threads=0):
     """The CPU step on a bounded sample of the same workload: the first scenes of the list with
-    the same number of agents per scene, the reference's threading model (all cores of the
-    affinity mask, capped at the box's share of 16), 20 warm-up steps, then timed steps."""
+    the same number of agents per scene, the reference's threading model (one worker per core),
+    20 warm-up steps, then timed steps.  Runs the compiled reference (oracle/_ref, built in the
+    development container from the reference's own sources) when that library is present, else
+    the restated oracle; which one is reported as `kind`."""
     import numpy as np
 
     from bps_nav_amd import episodes
     from oracle import bpo
-    lib = bpo.load_ref() or bpo.load_oracle()
-    cores = min(len(os.sched_getaffinity(0)), 16)
+    lib = bpo.load_ref()
+    if lib is None:
+        if require_ref:
+            print("bench.py: --require-ref given but oracle/_ref/libbpsref.so is not there", file=sys.stderr)
+            sys.exit(3)
+        log("oracle/_ref/libbpsref.so is not there: the CPU leg runs the restated oracle (kind \"port\")")
+        lib = bpo.load_oracle()
+    affinity = len(os.sched_getaffinity(0))
+    # a GPU box grants a job the CPU share of its GPU (16 cores of the host), whatever the
+    # affinity mask shows; more threads than that would be timed on borrowed cores
+    cores = threads if threads > 0 else min(affinity, 16)
     sample_scenes = min(len(workload), 16)
     n = sample_scenes * agents_per_scene
     t0 = time.time()
     sim = bpo.Sim(lib, workload[:sample_scenes], n, seed=seed, threads=cores)
     sim.reset()
-    log(f"cpu baseline ({lib.kind}) ready: {sample_scenes} scenes, {n} agents, {cores} threads, setup {time.time() - t0:.1f}s")
+    log(f"cpu baseline: {lib.path} (kind {lib.kind}); {sample_scenes} scenes, {n} agents, {cores} threads of {affinity} "
+        f"cores in the affinity mask, setup {time.time() - t0:.1f}s")
     rng = np.random.default_rng(77)
     for _ in range(20):
         sim.step(episodes.random_actions(rng, n, p_forward))
@@ -99,7 +143,8 @@ def cpu_baseline(workload, agents_per_scene, seed, p_forward, budget_s=20.0):
         elapsed1 += time.perf_counter() - t0
         steps1 += 1
     sim.close()
-    return {"value": n * steps / elapsed, "unit": "agent-steps/s", "cores": cores, "kind": lib.kind,
+    return {"value": n * steps / elapsed, "unit": "agent-steps/s", "cores": cores, "affinity_cores": affinity,
+            "kind": lib.kind, "library": os.path.relpath(lib.path, ROOT),
             "sample": f"first {sample_scenes} of the {len(workload)} scenes, {n} agents, 20 warm-up + {steps} timed steps",
             "single_thread_value": n1 * steps1 / elapsed1,
             "single_thread_sample": f"first 2 scenes, {n1} agents, 5 warm-up + {steps1} timed steps"}
@@ -128,6 +173,9 @@ def main():
     ap.add_argument("--agents", type=int, default=16384)
     ap.add_argument("--scenes", type=int, default=128)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--require-ref", action="store_true",
+                    help="exit with an error instead of timing the restated oracle when the compiled reference is missing")
+    ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU leg (default: affinity cores, at most 16)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, so a counter profile of this command holds a "
                          "kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -162,8 +210,7 @@ def main():
     gen.reset(0)
     for t in range(W):
         gen.step(0, actions[t])
-    c0 = gen.counters()
-    gen.set_profiling(True)
+    # headline: K steps, no per-kernel event recording inside the timed region
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for t in range(W, W + K):
@@ -171,41 +218,70 @@ def main():
         gen.step_end(0)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    gen.check_errors()
+    # second pass over the same actions' length with HIP events around every kernel (on the
+    # stream the kernels run on): per-kernel durations and the counters the roofline uses
+    P = min(K, 100)
+    extra = torch.multinomial(probs.expand(P, 4), N, replacement=True, generator=g).to(torch.int64).cuda()
+    c0 = gen.counters()
+    gen.set_profiling(True)
+    torch.cuda.synchronize()
+    tp = time.perf_counter()
+    for t in range(P):
+        gen.step_start(0, extra[t])
+        gen.step_end(0)
+    torch.cuda.synchronize()
+    profiled_elapsed = time.perf_counter() - tp
     gen.set_profiling(False)
     gen.check_errors()
     c1 = gen.counters()
     kt, profiled = gen.kernel_times()
+    assert profiled == P
     d = {k: c1[k] - c0[k] for k in c1 if k != "phase_cycles"}
     if any(c1["phase_cycles"]):
         ph = [a - b for a, b in zip(c1["phase_cycles"], c0["phase_cycles"])]
         log("A* phase cycles per expanded node (diagnostic build): " + " ".join(f"{v / max(1, d['astar_pops']):.0f}" for v in ph))
     dist = gen.get_infos(0)["distanceToGoal"].cpu().numpy()
-    log(f"timed {K} steps in {elapsed:.3f}s; per-kernel ms/step {json.dumps({k: round(v, 4) for k, v in kt.items()})}")
+    log(f"timed {K} steps in {elapsed:.3f}s ({elapsed / K * 1e3:.3f} ms/step); profiled pass: {P} steps, "
+        f"{profiled_elapsed / P * 1e3:.3f} ms/step, per-kernel ms/step {json.dumps({k: round(v, 4) for k, v in kt.items()})}")
+    K_ = K
+    K = P   # the counters below cover the profiled pass
     log(f"per step: {d['geodesic_queries'] / K:.0f} geodesic queries, {d['astar_pops'] / max(1, d['geodesic_queries']):.0f} "
         f"A* pops/query, corridor {d['corridor_polys'] / max(1, d['geodesic_queries']):.1f} polys/query, "
-        f"{d['resets'] / K:.1f} resets, {d.get('geo_link_spills', 0) / K:.0f} link spills, {d.get('geo_heap_spills', 0) / K:.0f} heap spills, {d.get('geo_long_path', 0) / K:.0f} on the large-LDS path; non-finite distances now: {int((~np.isfinite(dist)).sum())} of {N}")
+        f"{d['resets'] / K:.1f} resets, {d.get('geo_link_spills', 0) / K:.0f} link spills, {d.get('geo_heap_spills', 0) / K:.0f} heap spills, {d.get('geo_long_path', 0) / K:.0f} on the large-LDS path, {d.get('geo_tie_restarts', 0) / K:.0f} run again with the exact heap; non-finite distances now: {int((~np.isfinite(dist)).sum())} of {N}")
     # roofline of the dominant kernel (geodesic over the step's queries), HIP-event timed
     dominant = max(kt, key=kt.get)
     geo_bytes = BYTES_PER_CORRIDOR_POLY * d["corridor_polys"] + BYTES_PER_QUERY_ENDS * d["geodesic_queries"]
     geo_ms = kt["geodesic"]
     achieved = geo_bytes / K / (geo_ms * 1e-3) / 1e9 if geo_ms > 0 else 0.0
+    tracked = tracked_counters() if (N, S) == (16384, 128) else {}
+    expansions_per_s = d["astar_pops"] / K / (geo_ms * 1e-3) if geo_ms > 0 else 0.0
     roofline = {"bound": "hbm", "kernel": "k_geodesic", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": achieved / HBM_PEAK_GBS,
                 "measured_copy_gbs": copy_gbs, "frac_of_measured_copy": achieved / copy_gbs,
-                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (N, S) == (16384, 128) else None,
+                "traffic": float(tracked["traffic_bytes_per_launch"]) if "traffic_bytes_per_launch" in tracked else None,
+                "traffic_source": (os.path.relpath(COUNTER_SUMMARY, ROOT) + " @ " + tracked.get("commit", "?")) if tracked else None,
                 "dominant_kernel_by_time": dominant,
-                "kernel_ms_per_step": kt, "algorithmic_bytes_per_step": geo_bytes / K}
+                "kernel_ms_per_step": kt, "kernel_ms_steps": P, "algorithmic_bytes_per_step": geo_bytes / K,
+                "expanded_nodes_per_s": expansions_per_s}
+    if "valu_insts_per_expansion" in tracked:
+        # what actually bounds the kernel: vector instructions issued against what the chip can issue
+        v = float(tracked["valu_insts_per_expansion"])
+        roofline["valu_issue"] = {"insts_per_expanded_node": v, "achieved": expansions_per_s * v, "peak": VALU_ISSUE_PEAK,
+                                  "unit": "wavefront instructions/s", "frac": expansions_per_s * v / VALU_ISSUE_PEAK}
     gen.close()
+    K = K_
     result = {
         "metric": METRIC, "value": N * K / elapsed, "unit": "agent-steps/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": elapsed / K * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "C4: 16384 agents / 128 corridor-maze scenes (~30k polygons each), geodesic 15-40 m, "
-                               "P(forward)=0.8, auto-reset", "agents": N, "scenes": S, "parity": "bit-exact vs CPU oracle"},
+                               "P(forward)=0.8, auto-reset", "agents": N, "scenes": S},
         "roofline": roofline,
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(workload, N // S, seed, p_forward)
+        result["cpu_baseline"] = cpu_baseline(workload, N // S, seed, p_forward, require_ref=args.require_ref,
+                                              threads=args.cpu_threads)
         result["speedup_vs_cpu_baseline"] = result["value"] / result["cpu_baseline"]["value"]
     print(json.dumps(result), flush=True)
 

@@ -100,6 +100,7 @@ static_assert(sizeof(TileBVNode) == 16, "bv");
 static_assert(sizeof(TileOffMeshCon) == 36, "offmesh");
 
 inline int align4(int x) { return (x + 3) & ~3; }
+inline size_t align4(size_t x) { return (x + 3) & ~(size_t)3; }
 inline uint32_t nextPow2(uint32_t v) {
   v--; v |= v >> 1; v |= v >> 2; v |= v >> 4; v |= v >> 8; v |= v >> 16; v++;
   return v;

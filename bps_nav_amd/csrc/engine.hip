@@ -348,8 +348,6 @@ int bpsx_finalize(bpsx_sim* sim) {
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, sim->cfg.gpu_id));
   uint32_t per_cu = geodesic_blocks_per_cu();   // blocks of two wavefronts
-  // (for occupancy experiments: BPSX_GEO_WAVES_PER_CU overrides what the occupancy query says)
-  if (const char* e = getenv("BPSX_GEO_WAVES_PER_CU")) per_cu = (uint32_t)std::max(1, atoi(e) / 2);
   uint32_t blocks = (uint32_t)prop.multiProcessorCount * per_cu;
   if (blocks > sim->envs_per_group) blocks = sim->envs_per_group;
   sim->geo_blocks = std::max(1u, blocks);

@@ -117,7 +117,10 @@ BPSX_DEV uint32_t visit_cell(const AgentArrays& A, uint32_t gi, const float* pos
   const float d[3] = {pos[0] - ip[0], pos[1] - ip[1], pos[2] - ip[2]};
   float g[3];
   quat_rotate(iq, d, g);
-  const int32_t c0 = (int32_t)(g[0] / 1.0f), c1 = (int32_t)(g[1] / 1.0f), c2 = (int32_t)(g[2] / 1.0f);
+  // int(x) of the reference; for a value no int32 holds (or NaN) the x86 conversion the
+  // reference compiles to gives INT32_MIN, the GPU's would saturate: made explicit
+  auto cell = [](float x) { return (x > -2147483648.0f && x < 2147483648.0f) ? (int32_t)x : (int32_t)0x80000000; };
+  const int32_t c0 = cell(g[0] / 1.0f), c1 = cell(g[1] / 1.0f), c2 = cell(g[2] / 1.0f);
   int32_t* cells = A.exp_cells + (size_t)gi * A.cell_cap * 3;
   const uint32_t n = A.exp_count[gi];
   for (uint32_t i = 0; i < n; ++i)
@@ -458,9 +461,7 @@ __global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, 
 }
 
 #ifdef BPSX_QUERY_TRACE
-// diagnostic build: start/end time (100 MHz wall clock), nodes expanded and class of every query
-__device__ unsigned long long g_trace[1 << 17][4];
-__device__ unsigned int g_trace_n;
+#include "diag_trace.h"   // diagnostic build only: per-query trace buffer
 #endif
 // Work of one wavefront on one query, whichever instantiation g belongs to: the search, the
 // result and the agent's cost estimate.
@@ -702,16 +703,7 @@ void launch_random_points(const NavData& nav, uint32_t scene, const float* u, ui
 }
 
 #ifdef BPSX_QUERY_TRACE
-extern "C" __attribute__((visibility("default"))) int bpsx_debug_trace(unsigned long long* out, unsigned int max_rows) {
-  unsigned int n = 0;
-  (void)hipDeviceSynchronize();
-  (void)hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_trace_n), 4);
-  if (n > (1u << 17)) n = 1u << 17;
-  if (n > max_rows) n = max_rows;
-  if (out && n) (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), (size_t)n * 32);
-  const unsigned int zero = 0;
-  (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace_n), &zero, 4);
-  return (int)n;
-}
+#define BPSX_DIAG_TRACE_HOST
+#include "diag_trace.h"
 #endif
 }  // namespace bpsx

@@ -7,6 +7,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <initializer_list>
 
 #include "../../include/bpsx.h"
 #include "dt_format.h"
@@ -57,14 +58,22 @@ int parse_navmesh(const uint8_t* b, size_t n, HostScene* out) {
       h.maxLinkCount < 0 || h.detailVertCount < 0 || h.detailTriCount < 0 || h.bvNodeCount < 0)
     return fail(BPSX_E_INVAL, "navmesh: inconsistent tile header");
   if ((uint32_t)h.polyCount > (1u << polyBits)) return fail(BPSX_E_INVAL, "navmesh: polyCount exceeds maxPolys bits");
+  // the device tree names its right children and leaves in 16 bits, 0xffff marks a leaf
+  if (h.bvNodeCount > 0xfffe) return fail(BPSX_E_INVAL, "navmesh: more BV nodes than a tile of 32767 polygons can have");
+  // no section can hold more elements than the tile has bytes: checked before the counts are
+  // multiplied, and the sizes are computed in size_t
+  const size_t tileBytes = (size_t)th.dataSize;
+  for (const int count : {h.vertCount, h.polyCount, h.maxLinkCount, h.detailMeshCount, h.detailVertCount, h.detailTriCount,
+                          h.bvNodeCount})
+    if ((size_t)count > tileBytes) return fail(BPSX_E_INVAL, "navmesh: a section count exceeds the tile size");
   const size_t headerSize = align4(sizeof(TileHeader));
-  const size_t vertsSize = align4(12 * h.vertCount);
-  const size_t polysSize = align4(32 * h.polyCount);
-  const size_t linksSize = align4(12 * h.maxLinkCount);
-  const size_t dmSize = align4(12 * h.detailMeshCount);
-  const size_t dvSize = align4(12 * h.detailVertCount);
-  const size_t dtSize = align4(4 * h.detailTriCount);
-  const size_t bvSize = align4(16 * h.bvNodeCount);
+  const size_t vertsSize = align4((size_t)12 * (size_t)h.vertCount);
+  const size_t polysSize = align4((size_t)32 * (size_t)h.polyCount);
+  const size_t linksSize = align4((size_t)12 * (size_t)h.maxLinkCount);
+  const size_t dmSize = align4((size_t)12 * (size_t)h.detailMeshCount);
+  const size_t dvSize = align4((size_t)12 * (size_t)h.detailVertCount);
+  const size_t dtSize = align4((size_t)4 * (size_t)h.detailTriCount);
+  const size_t bvSize = align4((size_t)16 * (size_t)h.bvNodeCount);
   if (headerSize + vertsSize + polysSize + linksSize + dmSize + dvSize + dtSize + bvSize > (size_t)th.dataSize)
     return fail(BPSX_E_INVAL, "navmesh: tile sections exceed tile size");
   const float* verts = reinterpret_cast<const float*>(tileData + headerSize);

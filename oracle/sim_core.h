@@ -291,7 +291,9 @@ class Sim {
     const float d[3] = {e.pos[0] - e.initPos[0], e.pos[1] - e.initPos[1], e.pos[2] - e.initPos[2]};
     float g[3];
     quat_rotate(e.invInitRot, d, g);
-    const std::array<int, 3> cell = {(int)(g[0] / 1.0f), (int)(g[1] / 1.0f), (int)(g[2] / 1.0f)};
+    // int(x) as x86 converts it: INT32_MIN for NaN and for values no int32 holds
+    auto toCell = [](float x) { return (x > -2147483648.0f && x < 2147483648.0f) ? (int)x : (int)0x80000000; };
+    const std::array<int, 3> cell = {toCell(g[0] / 1.0f), toCell(g[1] / 1.0f), toCell(g[2] / 1.0f)};
     for (const auto& v : e.visited)
       if (v == cell) return;
     e.visited.push_back(cell);

@@ -629,3 +629,12 @@ def test_error_paths(oracle, torch_cuda):
         make_gen([(four, sc[0][1])], 8)
     with pytest.raises(RuntimeError, match="magic"):
         make_gen([(b"XXXX" + sc[0][0][4:], sc[0][1])], 8)
+    # hostile tile headers: counts that overflow 32-bit size arithmetic or the tree's 16-bit links
+    import struct
+    blob = bytearray(sc[0][0])
+    for off, val, msg in ((48 + 28, 0x7fffffff, "exceeds the tile size"), (48 + 48, 0x10000, "more BV nodes"),
+                          (48 + 32, 0x7ffffff0, "exceeds the tile size")):
+        bad = bytearray(blob)
+        struct.pack_into("<i", bad, off, val)
+        with pytest.raises(RuntimeError, match=msg):
+            make_gen([(bytes(bad), sc[0][1])], 8)
