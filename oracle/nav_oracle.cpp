@@ -6,6 +6,8 @@
 #include <cmath>
 #include <cstring>
 #include <limits>
+#include <queue>
+#include <algorithm>
 
 namespace orc {
 
@@ -902,7 +904,14 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
     if (outOfNodes) status |= ST_OUT_OF_NODES;
   }
   if (status != ST_SUCCESS || corridor_.empty()) return INF;
+  return corridorLength(start, end);
+}
 
+// findStraightPath over corridor_ and the summed length of its points (PathFinder.cpp:473-482,
+// 512-525; DetourNavMeshQuery.cpp:1765-1994).
+float Query::corridorLength(const NavPoint& start, const NavPoint& end) {
+  const Mesh& m = *mesh_;
+  const float INF = std::numeric_limits<float>::infinity();
   // ---- findStraightPath (options 0, at most 256 points)
   const int pathSize = (int)corridor_.size();
   counters.corridor_polys += (uint64_t)pathSize;
@@ -998,6 +1007,84 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
     prev = p;
   }
   return length;
+}
+
+// NOT a restatement of the reference: the goal-rooted distance-field formulation, for measuring
+// how far its distances are from findPath's.  A Dijkstra search from `start` (the goal point)
+// over the same graph A* searches (node = polygon, node position = midpoint of the portal
+// through which the polygon was first reached, edge cost = distance between node positions)
+// gives every polygon a parent towards the goal; the corridor of a query is the parent chain
+// from the end point's polygon, and the same string pulling gives the length.  The field is
+// kept while consecutive calls have the same start point.
+float Query::geodesicViaField(const NavPoint& start, const NavPoint& end) {
+  const Mesh& m = *mesh_;
+  const float INF = std::numeric_limits<float>::infinity();
+  {
+    const float* a = start.xyz;
+    const float* b = end.xyz;
+    const float d0 = a[0] - b[0], d1 = a[1] - b[1], d2 = a[2] - b[2];
+    const float dd = d0 * d0 + (d1 * d1 + d2 * d2);
+    const float aa = a[0] * a[0] + (a[1] * a[1] + a[2] * a[2]);
+    const float bb = b[0] * b[0] + (b[1] * b[1] + b[2] * b[2]);
+    const float mn = bb < aa ? bb : aa;
+    if (dd <= 1e-5f * 1e-5f * mn) return 0.0f;
+  }
+  int startIp, endIp;
+  if (!m.decode(start.ref, &startIp) || !m.decode(end.ref, &endIp)) return INF;
+  if (m.island[startIp] != m.island[endIp]) return INF;
+  if (!vfinite(start.xyz) || !vfinite(end.xyz)) return INF;
+  const int np = (int)m.polys.size();
+  if (field_.parent.size() != (size_t)np || field_.rootRef != start.ref || memcmp(field_.root, start.xyz, 12) != 0) {
+    field_.parent.assign((size_t)np, -2);   // -2 not reached, -1 root
+    field_.pos.assign((size_t)np * 3, 0.f);
+    field_.cost.assign((size_t)np, INF);
+    std::vector<uint8_t> closed((size_t)np, 0);
+    field_.rootRef = start.ref;
+    memcpy(field_.root, start.xyz, 12);
+    typedef std::pair<float, int> Item;
+    std::priority_queue<Item, std::vector<Item>, std::greater<Item>> open;
+    field_.parent[startIp] = -1;
+    field_.cost[startIp] = 0;
+    vcopy(&field_.pos[(size_t)startIp * 3], start.xyz);
+    open.push(Item(0.f, startIp));
+    while (!open.empty()) {
+      const Item it = open.top();
+      open.pop();
+      const int bi = it.second;
+      if (closed[bi] || it.first != field_.cost[bi]) continue;
+      closed[bi] = 1;
+      const Poly& bp = m.polys[bi];
+      for (uint32_t li = bp.firstLink; li != NULL_LINK; li = m.links[li].next) {
+        const uint32_t nref = m.links[li].ref;
+        if (!nref) continue;
+        const int ni = (int)(nref & ((1u << m.polyBits) - 1));
+        if (ni == field_.parent[bi] || !m.passFilter(m.polys[ni]) || closed[ni]) continue;
+        float* npos = &field_.pos[(size_t)ni * 3];
+        if (field_.parent[ni] == -2) {
+          float left[3], right[3];
+          if (portal_points(m, bi, nref, left, right)) {
+            npos[0] = (left[0] + right[0]) * 0.5f;
+            npos[1] = (left[1] + right[1]) * 0.5f;
+            npos[2] = (left[2] + right[2]) * 0.5f;
+          }
+        }
+        const float c = field_.cost[bi] + vdist(&field_.pos[(size_t)bi * 3], npos);
+        if (c < field_.cost[ni]) {
+          field_.cost[ni] = c;
+          field_.parent[ni] = bi;
+          open.push(Item(c, ni));
+        }
+      }
+    }
+  }
+  if (field_.parent[endIp] == -2) return INF;
+  corridor_.clear();
+  for (int c = endIp; c >= 0; c = field_.parent[c]) {
+    corridor_.push_back(m.refBase() | (uint32_t)c);
+    if ((int)corridor_.size() > MAX_PATH) return INF;   // the reference's corridor buffer holds 256 polygons
+  }
+  std::reverse(corridor_.begin(), corridor_.end());
+  return corridorLength(start, end);
 }
 
 bool Query::samplePoint(float u0, float s, float t, float* out_xyz, uint32_t* out_ref) {

@@ -73,6 +73,10 @@ class Query {
   NavPoint snapPoint(const float* pt);
   NavPoint tryStep(const NavPoint& start, const float* end);
   float geodesic(const NavPoint& start, const NavPoint& end);
+  // The distance-field formulation of the same query (NOT the reference's algorithm; only for
+  // measuring how far it is from geodesic()): parent chain of a goal-rooted Dijkstra search as
+  // the corridor, then the same string pulling.
+  float geodesicViaField(const NavPoint& start, const NavPoint& end);
   // Corridor of the last geodesic() that reached the funnel (polygon refs).
   const std::vector<uint32_t>& lastCorridor() const { return corridor_; }
   // Area-weighted pick: polygon by u0 over the float prefix sum of fan areas, then
@@ -86,6 +90,13 @@ class Query {
   const Mesh* mesh_;
   Impl* impl_;
   std::vector<uint32_t> corridor_;
+  float corridorLength(const NavPoint& start, const NavPoint& end);
+  struct Field {
+    uint32_t rootRef = 0;
+    float root[3] = {0, 0, 0};
+    std::vector<int> parent;
+    std::vector<float> pos, cost;
+  } field_;
 };
 
 }  // namespace orc

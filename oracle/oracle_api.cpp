@@ -85,6 +85,18 @@ BPO_API int bpo_nav_last_corridor(void* h, uint32_t* out, int max) {
   memcpy(out, c.data(), (size_t)n * 4);
   return (int)c.size();
 }
+// Distances of the goal-rooted distance-field formulation (orc::Query::geodesicViaField), for
+// the measurement of how far that formulation is from the reference's findPath.
+BPO_API void bpo_nav_geodesic_field(void* h, const float* sxyz, const uint32_t* sref, const float* exyz,
+                                    const uint32_t* eref, uint32_t n, float* out) {
+  orc::Query& q = *((ApiImpl<OracleBackend>::Nav*)h)->ctx->q[0];
+  for (uint32_t i = 0; i < n; ++i) {
+    orc::NavPoint a, b;
+    memcpy(a.xyz, &sxyz[(size_t)i * 3], 12); a.ref = sref[i];
+    memcpy(b.xyz, &exyz[(size_t)i * 3], 12); b.ref = eref[i];
+    out[i] = q.geodesicViaField(a, b);
+  }
+}
 BPO_API void bpo_random_point_in_convex_poly(const float* pts, int npts, float s, float t, float* out) {
   float areas[16];
   orc::random_point_in_convex_poly(pts, npts, areas, s, t, out);
