@@ -67,6 +67,18 @@ def test_batched_queries_match_oracle(oracle, torch_cuda, config):
     assert (gz == 0).all()
     gi = gen.geodesic(0, a[:4], np.zeros(4, np.uint32), b[:4], br[:4])
     assert np.isinf(gi).all()
+    # the vectors the compiled reference wrote for this scene (tests/golden/make_golden.py)
+    import os
+    import zlib
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", f"scene_c{config}.npz"))
+    assert zlib.crc32(blob) == int(g["crc"][0])
+    sx, sr = gen.snap_points(0, g["snap_in"])
+    assert np.array_equal(sr, g["snap_ref"]) and np.array_equal(common.bits(sx), common.bits(g["snap_xyz"]))
+    tx, tr = gen.try_steps(0, g["step_start"], g["snap_ref"], g["step_end"])
+    assert np.array_equal(tr, g["step_ref"]) and np.array_equal(common.bits(tx), common.bits(g["step_xyz"]))
+    p = g["geo_perm"]
+    gd = gen.geodesic(0, g["step_start"], g["snap_ref"], g["step_start"][p], g["snap_ref"][p])
+    assert np.array_equal(common.bits(gd), common.bits(g["geo_dist"])), "geodesics differ from the compiled reference's"
     gen.close()
 
 

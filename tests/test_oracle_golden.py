@@ -40,7 +40,7 @@ def test_handmade_mesh_queries(oracle, name):
         assert np.isinf(gd).any() and np.isfinite(gd).any()
 
 
-@pytest.mark.parametrize("config", [1, 2, 4])
+@pytest.mark.parametrize("config", [1, 2, 3, 4])
 def test_generated_scene_queries(oracle, config):
     g = np.load(os.path.join(GOLD, f"scene_c{config}.npz"))
     blob = scenes.config_scene(config, 0)
