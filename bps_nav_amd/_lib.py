@@ -13,7 +13,8 @@ LIB_PATH = os.environ.get("BPSX_LIBRARY") or os.path.join(_HERE, "libbpsx.so")
 class Config(C.Structure):
     _fields_ = [("num_environments", C.c_uint32), ("num_active_scenes", C.c_uint32),
                 ("double_buffered", C.c_uint32), ("reset_mode", C.c_uint32), ("seed", C.c_uint64),
-                ("gpu_id", C.c_int32), ("max_steps", C.c_uint32), ("task", C.c_uint32), ("scene_reserve", C.c_float)]
+                ("gpu_id", C.c_int32), ("max_steps", C.c_uint32), ("task", C.c_uint32), ("scene_reserve", C.c_float),
+                ("rotate_scenes", C.c_uint32), ("rotation_interval_ms", C.c_uint32)]
 
 
 class Outputs(C.Structure):
@@ -73,6 +74,9 @@ def lib():
             L.bpsx_finalize.argtypes = [C.c_void_p]
             L.bpsx_swap_scene.argtypes = [C.c_void_p, C.c_uint32, C.c_char_p, C.c_size_t, C.c_void_p, C.c_uint32]
             L.bpsx_swap_status.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint64)]
+            L.bpsx_active_scenes.argtypes = [C.c_void_p, C.c_void_p]
+            L.bpsx_rotation_log.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.POINTER(C.c_uint32)]
+            L.bpsx_swap_stats.argtypes = [C.c_void_p, C.POINTER(C.c_double)]
             L.bpsx_destroy.argtypes = [C.c_void_p]
             L.bpsx_destroy.restype = None
             L.bpsx_num_groups.argtypes = [C.c_void_p, C.POINTER(C.c_uint32)]

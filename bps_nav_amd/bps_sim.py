@@ -36,9 +36,11 @@ class InfoView:
 
 
 def load_dataset(dataset_path, asset_path):
-    """Reads `<dataset_path>/*.json.gz`, one scene per file, into [(navmesh_bytes, episodes)]
-    (Dataset::parseFile, simulator.cpp:190-336): start_position, start_rotation (x,y,z,w),
-    goals[0].position; the navmesh sits next to the scene asset with a .navmesh suffix."""
+    """Reads every `*.json.gz` of directory `dataset_path` (the reference is handed
+    `<split>/content`, env_utils.py:40-48), one scene per file, into [(navmesh_bytes, episodes)]
+    in file-name order (Dataset, simulator.cpp:190-336): start_position, start_rotation
+    (x,y,z,w), goals[0].position; the scene's navmesh is `<asset_path>/<scene_id up to its last
+    dot>.navmesh` (simulator.cpp:291-311).  A file without episodes adds no scene."""
     scenes = []
     for path in sorted(glob.glob(os.path.join(dataset_path, "*.json.gz"))):
         with gzip.open(path, "rt") as f:
@@ -47,7 +49,9 @@ def load_dataset(dataset_path, asset_path):
         if not eps:
             continue
         scene_id = eps[0]["scene_id"]
-        nav_path = os.path.join(asset_path, os.path.splitext(scene_id)[0] + ".navmesh")
+        if "." not in scene_id:
+            raise ValueError(f"{path}: invalid scene id {scene_id!r}")
+        nav_path = asset_path + "/" + scene_id[:scene_id.rfind(".")] + ".navmesh"
         with open(nav_path, "rb") as f:
             blob = f.read()
         rows = np.zeros((len(eps), 10), np.float32)
@@ -73,21 +77,25 @@ class PointNavRolloutGenerator:
 
     def __init__(self, dataset_path, asset_path, num_environments, num_active_scenes, num_workers=-1, gpu_id=0,
                  render_resolution=(64, 64), color=False, depth=False, double_buffered=False, seed=0,
-                 should_set_affinity=True, *, scenes=None, reset_mode=0, max_steps=0, scene_reserve=0.0):
+                 should_set_affinity=True, *, scenes=None, reset_mode=0, max_steps=0, scene_reserve=0.0, rotate=None,
+                 rotation_interval_ms=1000):
+        """`scenes` or the dataset directory may hold more scenes than num_active_scenes: the
+        library then picks the ones that start resident at random, on `seed`, and (rotate=True,
+        the default for a dataset directory, as in the reference) brings the others in over time,
+        loading at most one scene per rotation_interval_ms in a thread of its own."""
         self._L = _lib.lib()
         if not hasattr(self._L, "bpsx_create"):
             raise RuntimeError("libbpsx.so was built without the HIP engine")
+        if rotate is None:
+            rotate = scenes is None
         if scenes is None:
             scenes = load_dataset(dataset_path, asset_path)
-            if len(scenes) < num_active_scenes:
-                raise ValueError("dataset holds fewer scenes than num_active_scenes")
-            # the reference picks num_active_scenes of the dataset at random and rotates the
-            # rest in over time (simulator.cpp:1518-1534); here the first ones stay resident
-            scenes = scenes[:num_active_scenes]
+        if len(scenes) < num_active_scenes:
+            raise ValueError("dataset holds fewer scenes than num_active_scenes")
         self.gpu_id = gpu_id
         self.double_buffered = bool(double_buffered)
         cfg = _lib.Config(num_environments, num_active_scenes, int(self.double_buffered), reset_mode, seed, gpu_id,
-                          max_steps, self.TASK, scene_reserve)
+                          max_steps, self.TASK, scene_reserve, int(bool(rotate)), int(rotation_interval_ms))
         h = C.c_void_p()
         _lib.check(self._L.bpsx_create(C.byref(cfg), C.byref(h)))
         self._h = h
@@ -186,11 +194,30 @@ class PointNavRolloutGenerator:
 
     @property
     def swap_stats(self):
-        """(scene swaps completed per 100 steps taken, scenes in use, envs per scene) like
-        simulator.cpp:1412-1424."""
-        done = self.swap_status(0)[1]
-        steps = max(1, self.counters()["agent_steps"] // max(1, self.envs_per_group))
-        return (100.0 * done / steps, float(self.num_scenes), float(self.envs_per_group * self.num_groups) / self.num_scenes)
+        """(scene swaps completed per 100 env steps taken, scenes in use, envs per scene), the
+        last two summed over the groups, like simulator.cpp:1412-1424."""
+        out = (C.c_double * 3)()
+        _lib.check(self._L.bpsx_swap_stats(self._h, out))
+        return (out[0], out[1], out[2])
+
+    def active_scenes(self):
+        """Dataset index of the scene each slot's envs are on or are moving to."""
+        out = np.zeros(self.num_scenes, np.uint32)
+        _lib.check(self._L.bpsx_active_scenes(self._h, out.ctypes.data))
+        return out
+
+    def rotation_events(self):
+        """[(ordinal of the step_start that made the scene the slot's target, slot, dataset
+        index)] of the automatic swaps started since the last call; raises if the loader thread
+        failed on a scene."""
+        buf = np.zeros((64, 3), np.uint32)
+        n = C.c_uint32()
+        rows = []
+        while True:
+            _lib.check(self._L.bpsx_rotation_log(self._h, buf.ctypes.data, len(buf), C.byref(n)))
+            rows += [tuple(int(v) for v in r) for r in buf[:n.value]]
+            if n.value < len(buf):
+                return rows
 
     # ---- state and diagnostics for parity harnesses
     def get_state(self, group_idx):

@@ -5,10 +5,17 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cmath>
+#include <condition_variable>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
+#include <memory>
+#include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/bpsx.h"
@@ -117,11 +124,31 @@ struct SceneRanges {
 struct SceneSlot {
   uint32_t current = 0;         // scene-table entry of the resident scene
   uint32_t target = kNoSwap;    // entry of the scene being moved to, if a swap is in progress or just done
+  // automatic rotation (SceneSwapper, simulator.cpp:1063-1154)
+  uint32_t active_scene = 0;    // dataset index of the scene the slot's envs are on or are moving to
+  uint32_t load_entry = kNoSwap;          // scene-table entry the loader thread is filling / has filled
+  std::atomic<uint32_t> load_state{0};    // 0 none, 1 requested, 2 resident and ready, 3 failed
 };
+// One scene of the dataset as handed to bpsx_add_scene: kept as bytes while it is not resident.
+struct PoolScene {
+  std::vector<uint8_t> blob;
+  std::vector<float> episodes;
+  std::unique_ptr<HostScene> parsed;   // until finalize
+};
+
+// ---- counter-based stream of the scene choices (same integer arithmetic as the kernels' reset stream)
+static uint64_t mix64_host(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+static uint32_t scene_draw(uint64_t seed, uint64_t k) {
+  const uint64_t key = mix64_host(seed + 0x9E3779B97F4A7C15ull * 0x100000000ull + 0xD1B54A32D192ED03ull);
+  return (uint32_t)(mix64_host(key + 0x9E3779B97F4A7C15ull * (k + 1)) >> 32);
+}
 
 struct bpsx_sim {
   bpsx_config cfg{};
-  std::vector<HostScene> scenes;
   bool finalized = false;
   uint32_t num_groups = 1, envs_per_group = 0;
   // navmesh arrays
@@ -135,7 +162,24 @@ struct bpsx_sim {
   NavData nav{};
   Arena ar_poly, ar_bv, ar_tri, ar_dv, ar_ep;
   std::vector<SceneRanges> ranges;   // per scene-table entry
-  std::vector<SceneSlot> slots;
+  std::unique_ptr<SceneSlot[]> slots;
+  // dataset and automatic rotation
+  std::vector<PoolScene> pool;           // every scene added, in call order
+  std::vector<uint32_t> inactive;        // dataset indices not resident (simulator.cpp:1518-1534)
+  uint64_t scene_draws = 0;              // draws taken from the scene-choice stream
+  bool rotating = false;
+  std::mutex arena_mu;                   // the arenas are used by the loader thread too
+  std::thread loader;
+  std::mutex loader_mu;
+  std::condition_variable loader_cv;
+  std::deque<uint32_t> loader_requests;  // slots waiting for their next scene
+  bool loader_exit = false;
+  std::string loader_error;              // first failure of the loader thread (guarded by loader_mu)
+  hipStream_t upload_stream = nullptr;   // uploads of scenes that come in while the simulation runs
+  uint32_t* h_swap_remaining = nullptr;  // pinned copy of d_swap_remaining, refreshed by every step
+  bool remaining_fresh = false;
+  std::vector<uint32_t> rotation_log;    // (step ordinal, slot, dataset index) of swaps made available
+  uint64_t steps_started = 0, env_steps_taken = 0;
   uint32_t* d_swap_target = nullptr;
   uint32_t* d_swap_remaining = nullptr;
   uint64_t swaps_completed = 0;
@@ -220,47 +264,58 @@ int bpsx_add_scene(bpsx_sim* sim, const void* navmesh_bytes, size_t navmesh_size
   if (sim->finalized) return fail(BPSX_E_STATE, "add_scene: simulator already finalized");
   if (sim->cfg.reset_mode == BPSX_RESET_EPISODES && (!episodes || !num_episodes))
     return fail(BPSX_E_INVAL, "add_scene: episode-table reset needs at least one episode");
-  HostScene hs;
-  const int rc = parse_navmesh((const uint8_t*)navmesh_bytes, navmesh_size, &hs);
+  PoolScene ps;
+  ps.parsed.reset(new HostScene());
+  const int rc = parse_navmesh((const uint8_t*)navmesh_bytes, navmesh_size, ps.parsed.get());
   if (rc) return rc;
-  if (episodes && num_episodes) hs.episodes.assign(episodes, episodes + (size_t)num_episodes * 10);
-  hs.dev.ep_count = num_episodes;
-  sim->scenes.push_back(std::move(hs));
+  if (episodes && num_episodes) ps.episodes.assign(episodes, episodes + (size_t)num_episodes * 10);
+  ps.parsed->episodes = ps.episodes;
+  ps.parsed->dev.ep_count = num_episodes;
+  ps.blob.assign((const uint8_t*)navmesh_bytes, (const uint8_t*)navmesh_bytes + navmesh_size);
+  sim->pool.push_back(std::move(ps));
   return BPSX_OK;
 }
 
 // Places one parsed scene into the arrays and writes its scene-table entry.
-static int upload_scene(bpsx_sim* sim, HostScene& s, uint32_t entry) {
+// The copies go out on `st` and have completed when the function returns; other streams are
+// not waited for.
+static int upload_scene(bpsx_sim* sim, HostScene& s, uint32_t entry, hipStream_t st) {
   SceneRanges r;
   r.npoly = s.polys.size(); r.nbv = s.bv.size(); r.ntri = s.dtris.size() / 4; r.ndv = s.dverts.size() / 3;
   r.nep = s.episodes.size() / 10;
-  const bool a = sim->ar_poly.take(r.npoly, &r.poly);
-  const bool b = a && sim->ar_bv.take(r.nbv, &r.bv);
-  const bool c = b && sim->ar_tri.take(r.ntri, &r.tri);
-  const bool d = c && sim->ar_dv.take(r.ndv, &r.dv);
-  const bool e = d && sim->ar_ep.take(r.nep, &r.ep);
-  if (!e) {
-    if (a) sim->ar_poly.give(r.poly, r.npoly);
-    if (b) sim->ar_bv.give(r.bv, r.nbv);
-    if (c) sim->ar_tri.give(r.tri, r.ntri);
-    if (d) sim->ar_dv.give(r.dv, r.ndv);
-    return fail(BPSX_E_UNSUPPORTED, "scene does not fit the space reserved for scene rotation");
+  {
+    std::lock_guard<std::mutex> lk(sim->arena_mu);
+    const bool a = sim->ar_poly.take(r.npoly, &r.poly);
+    const bool b = a && sim->ar_bv.take(r.nbv, &r.bv);
+    const bool c = b && sim->ar_tri.take(r.ntri, &r.tri);
+    const bool d = c && sim->ar_dv.take(r.ndv, &r.dv);
+    const bool e = d && sim->ar_ep.take(r.nep, &r.ep);
+    if (!e) {
+      if (a) sim->ar_poly.give(r.poly, r.npoly);
+      if (b) sim->ar_bv.give(r.bv, r.nbv);
+      if (c) sim->ar_tri.give(r.tri, r.ntri);
+      if (d) sim->ar_dv.give(r.dv, r.ndv);
+      return fail(BPSX_E_UNSUPPORTED, "scene does not fit the space reserved for scene rotation");
+    }
   }
   r.used = true;
   s.dev.poly_base = (uint32_t)r.poly; s.dev.bv_base = (uint32_t)r.bv; s.dev.ep_base = (uint32_t)r.ep;
   s.dev.ep_count = (uint32_t)r.nep;
   for (auto& p : s.polys) { p.tri_base += (uint32_t)r.tri; p.dvert_base += (uint32_t)r.dv; }
-  HIP_TRY(hipMemcpy(sim->d_polys + r.poly, s.polys.data(), r.npoly * sizeof(PolyRec), hipMemcpyHostToDevice));
-  HIP_TRY(hipMemcpy(sim->d_aedges + r.poly * kNvp, s.aedges.data(), s.aedges.size() * sizeof(AEdge), hipMemcpyHostToDevice));
-  if (r.nbv) HIP_TRY(hipMemcpy(sim->d_bv + r.bv, s.bv.data(), r.nbv * sizeof(BVNodeDev), hipMemcpyHostToDevice));
-  if (r.ntri) HIP_TRY(hipMemcpy(sim->d_dtris + r.tri * 4, s.dtris.data(), s.dtris.size(), hipMemcpyHostToDevice));
-  if (r.ndv) HIP_TRY(hipMemcpy(sim->d_dverts + r.dv * 3, s.dverts.data(), s.dverts.size() * 4, hipMemcpyHostToDevice));
-  if (r.nep) HIP_TRY(hipMemcpy(sim->d_episodes + r.ep * 10, s.episodes.data(), s.episodes.size() * 4, hipMemcpyHostToDevice));
-  HIP_TRY(hipMemcpy(sim->d_scenes + entry, &s.dev, sizeof(SceneDev), hipMemcpyHostToDevice));
   sim->ranges[entry] = r;
+  const auto H2D = hipMemcpyHostToDevice;
+  HIP_TRY(hipMemcpyAsync(sim->d_polys + r.poly, s.polys.data(), r.npoly * sizeof(PolyRec), H2D, st));
+  HIP_TRY(hipMemcpyAsync(sim->d_aedges + r.poly * kNvp, s.aedges.data(), s.aedges.size() * sizeof(AEdge), H2D, st));
+  if (r.nbv) HIP_TRY(hipMemcpyAsync(sim->d_bv + r.bv, s.bv.data(), r.nbv * sizeof(BVNodeDev), H2D, st));
+  if (r.ntri) HIP_TRY(hipMemcpyAsync(sim->d_dtris + r.tri * 4, s.dtris.data(), s.dtris.size(), H2D, st));
+  if (r.ndv) HIP_TRY(hipMemcpyAsync(sim->d_dverts + r.dv * 3, s.dverts.data(), s.dverts.size() * 4, H2D, st));
+  if (r.nep) HIP_TRY(hipMemcpyAsync(sim->d_episodes + r.ep * 10, s.episodes.data(), s.episodes.size() * 4, H2D, st));
+  HIP_TRY(hipMemcpyAsync(sim->d_scenes + entry, &s.dev, sizeof(SceneDev), H2D, st));
+  HIP_TRY(hipStreamSynchronize(st));
   return BPSX_OK;
 }
 static void release_scene(bpsx_sim* sim, uint32_t entry) {
+  std::lock_guard<std::mutex> lk(sim->arena_mu);
   SceneRanges& r = sim->ranges[entry];
   if (!r.used) return;
   sim->ar_poly.give(r.poly, r.npoly); sim->ar_bv.give(r.bv, r.nbv); sim->ar_tri.give(r.tri, r.ntri);
@@ -268,17 +323,132 @@ static void release_scene(bpsx_sim* sim, uint32_t entry) {
   r = SceneRanges{};
 }
 
+// ---- automatic scene rotation.  Counterpart of SceneSwapper + BackgroundSceneLoader
+// (simulator.cpp:361-551, 1063-1154): a loader thread parses the next scene of a slot and
+// uploads it on a stream of its own while the simulation steps; step_start makes a scene that
+// has become resident the slot's target (preStep), the envs move over when their episodes end,
+// and step_end, once none is left on the old scene, frees it and draws the slot's next scene
+// from the scenes that are not resident (postStep / startSceneSwap).
+static void loader_loop(bpsx_sim* sim) {
+  (void)hipSetDevice(sim->cfg.gpu_id);
+  auto last = std::chrono::steady_clock::now() - std::chrono::hours(1);
+  for (;;) {
+    uint32_t slot;
+    {
+      std::unique_lock<std::mutex> lk(sim->loader_mu);
+      sim->loader_cv.wait(lk, [&] { return sim->loader_exit || !sim->loader_requests.empty(); });
+      if (sim->loader_exit) return;
+      slot = sim->loader_requests.front();
+      sim->loader_requests.pop_front();
+    }
+    // at most one load per interval (the reference's RATE_LIMIT of one second, simulator.cpp:545-548)
+    const auto gap = std::chrono::milliseconds(sim->cfg.rotation_interval_ms);
+    const auto now = std::chrono::steady_clock::now();
+    if (now - last < gap) {
+      std::unique_lock<std::mutex> lk(sim->loader_mu);
+      sim->loader_cv.wait_for(lk, gap - (now - last), [&] { return sim->loader_exit; });
+      if (sim->loader_exit) return;
+    }
+    last = std::chrono::steady_clock::now();
+    SceneSlot& sl = sim->slots[slot];
+    const PoolScene& ps = sim->pool[sl.active_scene];
+    HostScene hs;
+    int rc = parse_navmesh(ps.blob.data(), ps.blob.size(), &hs);
+    if (!rc) {
+      hs.episodes = ps.episodes;
+      rc = upload_scene(sim, hs, sl.load_entry, sim->upload_stream);
+    }
+    if (rc) {
+      std::lock_guard<std::mutex> lk(sim->loader_mu);
+      if (sim->loader_error.empty())
+        sim->loader_error = "scene " + std::to_string(sl.active_scene) + " for slot " + std::to_string(slot) + ": " + last_error_message();
+      sl.load_state.store(3, std::memory_order_release);
+    } else {
+      sl.load_state.store(2, std::memory_order_release);
+    }
+  }
+}
+// SceneSwapper::startSceneSwap (simulator.cpp:1093-1106): a scene that is not resident, drawn
+// uniformly, changes places with the slot's scene and is sent to the loader.
+static void start_scene_swap(bpsx_sim* sim, uint32_t slot) {
+  if (sim->inactive.empty()) return;
+  SceneSlot& sl = sim->slots[slot];
+  const uint32_t r = scene_draw(sim->cfg.seed, sim->scene_draws++);
+  const uint32_t pos = (uint32_t)(((uint64_t)r * (uint64_t)sim->inactive.size()) >> 32);
+  std::swap(sim->inactive[pos], sl.active_scene);
+  const uint32_t S = sim->cfg.num_active_scenes;
+  sl.load_entry = sl.current < S ? slot + S : slot;   // the slot's other scene-table entry
+  sl.load_state.store(1, std::memory_order_release);
+  {
+    std::lock_guard<std::mutex> lk(sim->loader_mu);
+    sim->loader_requests.push_back(slot);
+  }
+  sim->loader_cv.notify_one();
+}
+// SceneSwapper::preStep: scenes that have become resident are what their slots' envs move to
+// from this step on.  The switch is made by a kernel on the step's stream, in order with the step.
+static int rotation_pre_step(bpsx_sim* sim, hipStream_t st) {
+  const uint32_t S = sim->cfg.num_active_scenes, per = sim->cfg.num_environments / S;
+  for (uint32_t slot = 0; slot < S; ++slot) {
+    SceneSlot& sl = sim->slots[slot];
+    if (sl.load_state.load(std::memory_order_acquire) != 2) continue;
+    sl.load_state.store(0, std::memory_order_relaxed);
+    sl.target = sl.load_entry;
+    launch_set_swap(sim->d_swap_target, sim->d_swap_remaining, slot, sl.target, per, st);
+    HIP_TRY(hipGetLastError());
+    sim->h_swap_remaining[slot] = per;
+    sim->rotation_log.push_back((uint32_t)sim->steps_started);
+    sim->rotation_log.push_back(slot);
+    sim->rotation_log.push_back(sl.active_scene);
+  }
+  return BPSX_OK;
+}
+// SceneSwapper::postStep: a slot whose envs have all moved gives its old scene's space back and
+// starts loading its next scene.
+static void rotation_post_step(bpsx_sim* sim) {
+  const uint32_t S = sim->cfg.num_active_scenes;
+  for (uint32_t slot = 0; slot < S; ++slot) {
+    SceneSlot& sl = sim->slots[slot];
+    if (sl.target == kNoSwap || sl.target == sl.current || sim->h_swap_remaining[slot] != 0) continue;
+    release_scene(sim, sl.current);
+    sl.current = sl.target;   // the device keeps the target: envs already on it ignore it
+    sim->swaps_completed++;
+    if (sim->rotating) start_scene_swap(sim, slot);
+  }
+}
+
 int bpsx_finalize(bpsx_sim* sim) {
   if (!sim) return fail(BPSX_E_INVAL, "finalize: null simulator");
   if (sim->finalized) return fail(BPSX_E_STATE, "finalize: called twice");
-  if (sim->scenes.size() != sim->cfg.num_active_scenes)
-    return fail(BPSX_E_INVAL, "finalize: number of scenes added differs from num_active_scenes");
+  const uint32_t S = sim->cfg.num_active_scenes;
+  if (sim->pool.size() < S) return fail(BPSX_E_INVAL, "finalize: fewer scenes added than num_active_scenes");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  // ---- which scenes of the dataset start resident: selection sampling over the dataset in
+  // order, like simulator.cpp:1518-1534 (there on the generator's mt19937, here on the
+  // counter-based stream): scene i is taken when u * (D - i) < scenes still to take.  With as
+  // many scenes as slots every scene is taken, in order.
+  {
+    const uint32_t D = (uint32_t)sim->pool.size();
+    std::vector<uint32_t> active;
+    uint32_t i = 0;
+    for (; i < D && active.size() < S; ++i) {
+      const float weight = (float)(scene_draw(sim->cfg.seed, sim->scene_draws++) >> 8) * (1.0f / 16777216.0f);
+      if (weight * (float)(D - i) < (float)(S - (uint32_t)active.size())) active.push_back(i);
+      else sim->inactive.push_back(i);
+    }
+    for (; i < D; ++i) sim->inactive.push_back(i);
+    sim->slots.reset(new SceneSlot[S]);
+    for (uint32_t k = 0; k < S; ++k) sim->slots[k].active_scene = active[k];
+  }
   // ---- navmesh arrays: every scene is a range of each array; room for scene rotation
   size_t npoly = 0, nbv = 0, ntri = 0, ndv = 0, nep = 0, mpoly = 0, mbv = 0, mtri = 0, mdv = 0, mep = 0;
-  for (auto& s : sim->scenes) {
+  for (uint32_t k = 0; k < S; ++k) {
+    const HostScene& s = *sim->pool[sim->slots[k].active_scene].parsed;
     npoly += s.polys.size(); nbv += s.bv.size(); ntri += s.dtris.size() / 4; ndv += s.dverts.size() / 3;
     nep += s.episodes.size() / 10;
+  }
+  for (auto& ps : sim->pool) {   // any scene of the dataset may come in later
+    const HostScene& s = *ps.parsed;
     mpoly = std::max(mpoly, s.polys.size()); mbv = std::max(mbv, s.bv.size()); mtri = std::max(mtri, s.dtris.size() / 4);
     mdv = std::max(mdv, s.dverts.size() / 3); mep = std::max(mep, s.episodes.size() / 10);
   }
@@ -289,7 +459,6 @@ int bpsx_finalize(bpsx_sim* sim) {
                cep = room(nep, mep);
   if (cpoly > 0xfffffff0ull || ctri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
   int rc;
-  const uint32_t S = sim->cfg.num_active_scenes;
   if ((rc = sim->alloc(&sim->d_polys, cpoly))) return rc;
   if ((rc = sim->alloc(&sim->d_aedges, cpoly * kNvp))) return rc;
   if ((rc = sim->alloc(&sim->d_bv, cbv))) return rc;
@@ -300,18 +469,24 @@ int bpsx_finalize(bpsx_sim* sim) {
   if ((rc = sim->alloc(&sim->d_swap_target, S)) || (rc = sim->alloc(&sim->d_swap_remaining, S))) return rc;
   sim->ar_poly.init(cpoly); sim->ar_bv.init(cbv); sim->ar_tri.init(ctri); sim->ar_dv.init(cdv); sim->ar_ep.init(cep);
   sim->ranges.assign(2 * (size_t)S, SceneRanges{});
-  sim->slots.assign(S, SceneSlot{});
   sim->nav = NavData{sim->d_polys, sim->d_aedges, sim->d_bv, sim->d_dtris, sim->d_dverts, sim->d_scenes, sim->d_episodes};
   {
     std::vector<uint32_t> none(S, kNoSwap);
     HIP_TRY(hipMemcpy(sim->d_swap_target, none.data(), (size_t)S * 4, hipMemcpyHostToDevice));
   }
+  HIP_TRY(hipStreamCreateWithFlags(&sim->upload_stream, hipStreamNonBlocking));
+  HIP_TRY(hipHostMalloc((void**)&sim->h_swap_remaining, (size_t)S * 4, hipHostMallocDefault));
+  memset(sim->h_swap_remaining, 0, (size_t)S * 4);
   for (uint32_t i = 0; i < S; ++i) {
     sim->slots[i].current = i;
-    if ((rc = upload_scene(sim, sim->scenes[i], i))) return rc;
+    if ((rc = upload_scene(sim, *sim->pool[sim->slots[i].active_scene].parsed, i, sim->upload_stream))) return rc;
   }
-  sim->scenes.clear();   // the host copies are not needed any more
-  sim->scenes.shrink_to_fit();
+  // the parsed copies are not needed any more; the bytes stay only if scenes will rotate
+  sim->rotating = sim->cfg.rotate_scenes && !sim->inactive.empty();
+  for (auto& ps : sim->pool) {
+    ps.parsed.reset();
+    if (!sim->rotating) { ps.blob.clear(); ps.blob.shrink_to_fit(); ps.episodes.clear(); ps.episodes.shrink_to_fit(); }
+  }
 
   // ---- agent state
   const size_t N = sim->cfg.num_environments;
@@ -370,6 +545,11 @@ int bpsx_finalize(bpsx_sim* sim) {
   // that the entry point itself makes no set-up call
   if ((rc = static_scratch_setup(sim->cfg.gpu_id))) return rc;
   sim->finalized = true;
+  if (sim->rotating) {
+    // every slot starts loading its next scene right away (simulator.cpp:1573)
+    sim->loader = std::thread(loader_loop, sim);
+    for (uint32_t i = 0; i < S; ++i) start_scene_swap(sim, i);
+  }
   return BPSX_OK;
 }
 
@@ -379,6 +559,16 @@ void bpsx_destroy(bpsx_sim* sim) {
     (void)hipSetDevice(sim->cfg.gpu_id);
     (void)hipDeviceSynchronize();
   }
+  if (sim->loader.joinable()) {
+    {
+      std::lock_guard<std::mutex> lk(sim->loader_mu);
+      sim->loader_exit = true;
+    }
+    sim->loader_cv.notify_all();
+    sim->loader.join();
+  }
+  if (sim->upload_stream) (void)hipStreamDestroy(sim->upload_stream);
+  if (sim->h_swap_remaining) (void)hipHostFree(sim->h_swap_remaining);
   for (auto& g : sim->groups) {
     if (g.h_actions) (void)hipHostFree(g.h_actions);
     if (g.done) (void)hipEventDestroy(g.done);
@@ -432,12 +622,22 @@ int bpsx_step_start(bpsx_sim* sim, uint32_t group, const int64_t* actions, int a
     HIP_TRY(hipMemcpyAsync(g.d_actions, g.h_actions, (size_t)sim->envs_per_group * sizeof(int64_t), hipMemcpyHostToDevice, st));
     d_act = g.d_actions;
   }
+  if ((rc = rotation_pre_step(sim, st))) return rc;
   g.profiled = sim->profiling;
   launch_step(sim->nav, sim->A, g.Q, sim->params(group), d_act, sim->d_slots, sim->geo_blocks, sim->snap_blocks, st,
               g.profiled ? g.ev : nullptr);
   HIP_TRY(hipGetLastError());
+  // how many envs of each slot are still on a scene that is leaving: read back with the step
+  sim->remaining_fresh = false;
+  for (uint32_t slot = 0; slot < sim->cfg.num_active_scenes && !sim->remaining_fresh; ++slot)
+    sim->remaining_fresh = sim->slots[slot].target != kNoSwap && sim->slots[slot].target != sim->slots[slot].current;
+  if (sim->remaining_fresh)
+    HIP_TRY(hipMemcpyAsync(sim->h_swap_remaining, sim->d_swap_remaining, (size_t)sim->cfg.num_active_scenes * 4,
+                           hipMemcpyDeviceToHost, st));
   HIP_TRY(hipEventRecord(g.done, st));
   g.in_flight = true;
+  sim->steps_started++;
+  sim->env_steps_taken += sim->envs_per_group;
   return BPSX_OK;
 }
 
@@ -449,6 +649,7 @@ int bpsx_step_end(bpsx_sim* sim, uint32_t group) {
   if (!g.in_flight) return fail(BPSX_E_STATE, "step_end: no step in flight for this group");
   HIP_TRY(hipEventSynchronize(g.done));
   g.in_flight = false;
+  if (sim->remaining_fresh && sim->rotating) rotation_post_step(sim);
   if (g.profiled) {
     for (int k = 0; k < BPSX_NUM_KERNELS; ++k) {
       float ms = 0;
@@ -563,8 +764,10 @@ int bpsx_swap_scene(bpsx_sim* sim, uint32_t slot, const void* navmesh_bytes, siz
     return fail(BPSX_E_INVAL, "swap_scene: episode-table reset needs at least one episode");
   for (auto& g : sim->groups)
     if (g.in_flight) return fail(BPSX_E_STATE, "swap_scene: a step is in flight");
+  if (sim->rotating) return fail(BPSX_E_STATE, "swap_scene: this simulator rotates its scenes by itself");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
-  HIP_TRY(hipDeviceSynchronize());   // nothing may still read a scene that is about to leave
+  // no step is in flight and every earlier one was waited for in step_end: nothing reads the
+  // scene that may leave now, and the upload below runs on a stream of its own
   uint32_t remaining = 0;
   int rc = settle_slot(sim, slot, &remaining);
   if (rc) return rc;
@@ -575,7 +778,7 @@ int bpsx_swap_scene(bpsx_sim* sim, uint32_t slot, const void* navmesh_bytes, siz
   SceneSlot& sl = sim->slots[slot];
   const uint32_t S = sim->cfg.num_active_scenes;
   const uint32_t entry = sl.current < S ? slot + S : slot;   // the slot's other table entry
-  if ((rc = upload_scene(sim, hs, entry))) return rc;
+  if ((rc = upload_scene(sim, hs, entry, sim->upload_stream))) return rc;
   const uint32_t per = sim->cfg.num_environments / S;
   HIP_TRY(hipMemcpy(sim->d_swap_remaining + slot, &per, 4, hipMemcpyHostToDevice));
   HIP_TRY(hipMemcpy(sim->d_swap_target + slot, &entry, 4, hipMemcpyHostToDevice));
@@ -589,12 +792,70 @@ int bpsx_swap_status(bpsx_sim* sim, uint32_t slot, uint32_t* envs_remaining, uin
   for (auto& g : sim->groups)
     if (g.in_flight) return fail(BPSX_E_STATE, "swap_status: a step is in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
-  HIP_TRY(hipDeviceSynchronize());
   uint32_t remaining = 0;
-  const int rc = settle_slot(sim, slot, &remaining);
-  if (rc) return rc;
+  if (sim->rotating) {
+    // as of the last step (step_end keeps the count and completes swaps by itself)
+    const SceneSlot& sl = sim->slots[slot];
+    remaining = (sl.target != kNoSwap && sl.target != sl.current) ? sim->h_swap_remaining[slot] : 0;
+  } else {
+    // every slot is brought up to date, so that completed swaps are counted and their old
+    // scenes' space is released whichever slot is asked about
+    for (uint32_t k = 0; k < sim->cfg.num_active_scenes; ++k) {
+      uint32_t rem = 0;
+      const int rc = settle_slot(sim, k, &rem);
+      if (rc) return rc;
+      if (k == slot) remaining = rem;
+    }
+  }
   if (envs_remaining) *envs_remaining = remaining;
   if (swaps_completed) *swaps_completed = sim->swaps_completed;
+  return BPSX_OK;
+}
+
+int bpsx_active_scenes(bpsx_sim* sim, uint32_t* out) {
+  if (!sim || !sim->finalized || !out) return fail(BPSX_E_STATE, "active_scenes: simulator not finalized");
+  for (uint32_t k = 0; k < sim->cfg.num_active_scenes; ++k) {
+    const SceneSlot& sl = sim->slots[k];
+    // while the slot's next scene is still loading, its envs are on the scene that was drawn before:
+    // that scene's index went back to the scenes that are not resident only in name
+    out[k] = sl.active_scene;
+  }
+  return BPSX_OK;
+}
+
+int bpsx_rotation_log(bpsx_sim* sim, uint32_t* out, uint32_t max_rows, uint32_t* num_rows) {
+  if (!sim || !sim->finalized || !num_rows) return fail(BPSX_E_STATE, "rotation_log: simulator not finalized");
+  const uint32_t have = (uint32_t)(sim->rotation_log.size() / 3);
+  const uint32_t n = have < max_rows ? have : max_rows;
+  if (n && !out) return fail(BPSX_E_INVAL, "rotation_log: null buffer");
+  if (n) memcpy(out, sim->rotation_log.data(), (size_t)n * 12);
+  sim->rotation_log.erase(sim->rotation_log.begin(), sim->rotation_log.begin() + (long)n * 3);
+  *num_rows = n;
+  std::lock_guard<std::mutex> lk(sim->loader_mu);
+  if (!sim->loader_error.empty()) return fail(BPSX_E_INVAL, "scene rotation: loading failed: " + sim->loader_error);
+  return BPSX_OK;
+}
+
+int bpsx_swap_stats(bpsx_sim* sim, double* out) {
+  if (!sim || !sim->finalized || !out) return fail(BPSX_E_STATE, "swap_stats: simulator not finalized");
+  const uint32_t S = sim->cfg.num_active_scenes, per = sim->cfg.num_environments / S;
+  out[0] = sim->env_steps_taken ? 100.0 * (double)sim->swaps_completed / (double)sim->env_steps_taken : 0.0;
+  // scenes in use and mean envs per scene, summed over the groups like simulator.cpp:1412-1424
+  double scenes = 0, mean = 0;
+  const uint32_t per_group = S / sim->num_groups;
+  for (uint32_t g = 0; g < sim->num_groups; ++g) {
+    uint32_t in_use = 0;
+    for (uint32_t k = g * per_group; k < (g + 1) * per_group; ++k) {
+      const SceneSlot& sl = sim->slots[k];
+      const bool moving = sl.target != kNoSwap && sl.target != sl.current;
+      const uint32_t rem = moving ? sim->h_swap_remaining[k] : 0;
+      in_use += (moving && rem > 0 && rem < per) ? 2u : 1u;
+    }
+    scenes += in_use;
+    mean += (double)sim->envs_per_group / (double)in_use;
+  }
+  out[1] = scenes;
+  out[2] = mean;
   return BPSX_OK;
 }
 

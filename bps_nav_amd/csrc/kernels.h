@@ -54,6 +54,9 @@ void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,
                           hipStream_t st);
 
+void launch_set_swap(uint32_t* swap_target, uint32_t* swap_remaining, uint32_t slot, uint32_t target, uint32_t envs,
+                     hipStream_t st);
+
 // Wavefronts of the A* kernel that one compute unit holds at once (bounded by their LDS).
 uint32_t geodesic_blocks_per_cu();
 

@@ -131,6 +131,14 @@ BPSX_DEV uint32_t visit_cell(const AgentArrays& A, uint32_t gi, const float* pos
   return n + 1;
 }
 
+// makes scene-table entry `target` what the envs of `slot` move to when their episodes end
+__global__ void k_set_swap(uint32_t* swap_target, uint32_t* swap_remaining, uint32_t slot, uint32_t target, uint32_t envs) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    swap_remaining[slot] = envs;
+    swap_target[slot] = target;
+  }
+}
+
 __global__ void k_clear_queues(StepQueues Q) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     for (int c = 0; c < kGeoClasses; ++c) Q.counts[kQGeo + c] = 0;
@@ -696,6 +704,10 @@ void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz
   // one class only: stride 0 puts its queries at the start of the buffer
   launch_geodesic(nav, qbuf, 0, &count_head[0], &count_head[kGeoClasses], &count_head[kGeoClasses + 1], out, nullptr, slots,
                   geo_blocks, counters, st);
+}
+void launch_set_swap(uint32_t* swap_target, uint32_t* swap_remaining, uint32_t slot, uint32_t target, uint32_t envs,
+                     hipStream_t st) {
+  hipLaunchKernelGGL(k_set_swap, dim3(1), dim3(64), 0, st, swap_target, swap_remaining, slot, target, envs);
 }
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,
                           hipStream_t st) {

@@ -74,6 +74,10 @@ typedef struct bpsx_config {
   uint32_t task;              /* BPSX_TASK_*                                               */
   float scene_reserve;        /* space for scene rotation: capacity of the navmesh arrays as
                                  a multiple of the initial scenes' total size; 0 => 3      */
+  uint32_t rotate_scenes;     /* 1 => when more scenes were added than are resident, rotate
+                                 through them by itself (SceneSwapper, simulator.cpp:1063-1154) */
+  uint32_t rotation_interval_ms; /* least time between two scene loads of the loader thread
+                                 (the reference's RATE_LIMIT is 1000, simulator.cpp:545-548)  */
 } bpsx_config;
 
 /* Output tensors of one group, device pointers that stay valid and fixed for the
@@ -103,10 +107,13 @@ typedef struct bpsx_state {
 
 /* ---- simulator lifecycle (RolloutGenerator ctor, simulator.cpp:1463-1617) ---- */
 int bpsx_create(const bpsx_config *cfg, bpsx_sim **out);
-/* Adds one scene: the bytes of a habitat ".navmesh" file (PathFinder::loadNavMesh,
+/* Adds one scene of the dataset: the bytes of a habitat ".navmesh" file (PathFinder::loadNavMesh,
  * PathFinder.cpp:330-408) and its episode table, E rows of 10 floats
  * {start xyz, start rotation xyzw, goal xyz} (struct Episode, simulator.cpp:83-87).
- * Host pointers; copied. Scenes get indices in call order. */
+ * Host pointers; copied. Scenes get dataset indices in call order.  At least
+ * num_active_scenes scenes must be added; of more, finalize picks the ones that start
+ * resident at random (Dataset + the selection loop of simulator.cpp:1518-1534, on the
+ * simulator's seed) and, with bpsx_config.rotate_scenes, the others come in over time. */
 int bpsx_add_scene(bpsx_sim *sim, const void *navmesh_bytes, size_t navmesh_size,
                    const float *episodes, uint32_t num_episodes);
 /* Uploads all scenes, assigns envs to scenes in contiguous blocks of
@@ -119,8 +126,8 @@ void bpsx_destroy(bpsx_sim *sim);
  * on every env of that slot moves to the new scene, with its episode table, when its episode
  * ends (not on an explicit reset); the old scene stays resident meanwhile.  One swap per slot
  * at a time: BPSX_E_STATE while envs are still on the old scene (the reference's
- * canSwapScene()).  The reference loads in a background thread and picks the scene at random;
- * here the caller chooses the scene and the call returns when it is resident.  Must not be
+ * canSwapScene()).  This is the caller-driven form: the caller chooses the scene and the call
+ * returns when it is resident (uploaded on a stream of the library's own).  Must not be
  * called between step_start and step_end.  BPSX_E_UNSUPPORTED if the scene does not fit the
  * space reserved at finalize (bpsx_config.scene_reserve). */
 int bpsx_swap_scene(bpsx_sim *sim, uint32_t slot, const void *navmesh_bytes, size_t navmesh_size,
@@ -128,6 +135,22 @@ int bpsx_swap_scene(bpsx_sim *sim, uint32_t slot, const void *navmesh_bytes, siz
 /* Envs of the slot that are still on the old scene (0: no swap in progress), and the number
  * of swaps completed over all slots since creation (swap_stats, simulator.cpp:1412-1424). */
 int bpsx_swap_status(bpsx_sim *sim, uint32_t slot, uint32_t *envs_remaining, uint64_t *swaps_completed);
+
+/* Automatic rotation (bpsx_config.rotate_scenes): a loader thread inside the library parses and
+ * uploads the next scene of a slot on a stream of its own while the simulation steps;
+ * step_start makes a scene that has become resident the slot's target, step_end frees the old
+ * scene once every env has left it and draws the slot's next scene uniformly from the scenes
+ * that are not resident (startSceneSwap / preStep / postStep, simulator.cpp:1093-1128).
+ * bpsx_swap_scene is refused on such a simulator.
+ * active_scenes: dataset index of the scene each slot's envs are on or are moving to.
+ * rotation_log: rows {ordinal of the step_start that made the scene the slot's target, slot,
+ * dataset index} of the swaps started since the last call (a parity harness repeats them on
+ * its own simulator); also returns BPSX_E_INVAL once if the loader thread failed on a scene.
+ * swap_stats: {swaps completed per 100 env steps, scenes in use, envs per scene} as the
+ * reference's swap_stats property computes them (simulator.cpp:1412-1424). */
+int bpsx_active_scenes(bpsx_sim *sim, uint32_t *out /* [num_active_scenes] */);
+int bpsx_rotation_log(bpsx_sim *sim, uint32_t *out /* [max_rows][3] */, uint32_t max_rows, uint32_t *num_rows);
+int bpsx_swap_stats(bpsx_sim *sim, double *out /* [3] */);
 
 /* ---- stepping (simulator.cpp:1377-1410) ---- */
 int bpsx_num_groups(const bpsx_sim *sim, uint32_t *out);

@@ -21,9 +21,9 @@ def torch_cuda():
     return torch
 
 
-def make_gen(sc, n, **kw):
+def make_gen(sc, n, num_active_scenes=None, **kw):
     from bps_nav_amd.bps_sim import PointNavRolloutGenerator
-    return PointNavRolloutGenerator("", "", n, len(sc), scenes=sc, **kw)
+    return PointNavRolloutGenerator("", "", n, num_active_scenes or len(sc), scenes=sc, **kw)
 
 
 @pytest.mark.parametrize("config", [1, 2, 3, 4])
@@ -592,6 +592,128 @@ def test_scene_rotation_parity(oracle, torch_cuda):
     assert gen.swap_status(0)[1] >= 6, "swaps did not complete"
     assert gen.swap_stats[0] > 0
     gen.check_errors()
+    gen.close()
+
+
+def write_dataset(root, pool):
+    """A dataset directory in the reference's layout (simulator.cpp:190-336, env_utils.py:40-48):
+    <root>/content/<scene>.json.gz with that scene's episodes, navmeshes under <root>/assets."""
+    import gzip
+    import json
+    import os
+    os.makedirs(os.path.join(root, "content"))
+    os.makedirs(os.path.join(root, "assets", "plans"))
+    for i, (blob, eps) in enumerate(pool):
+        with open(os.path.join(root, "assets", "plans", f"s{i:02d}.navmesh"), "wb") as f:
+            f.write(blob)
+        rows = [{"episode_id": str(k), "scene_id": f"plans/s{i:02d}.glb", "start_position": [float(v) for v in e[0:3]],
+                 "start_rotation": [float(v) for v in e[3:7]], "goals": [{"position": [float(v) for v in e[7:10]]}]}
+                for k, e in enumerate(eps)]
+        with gzip.open(os.path.join(root, "content", f"s{i:02d}.json.gz"), "wt") as f:
+            json.dump({"episodes": rows}, f)
+    return os.path.join(root, "content"), os.path.join(root, "assets")
+
+
+class ScenePolicy:
+    """Independent restatement of which scenes the reference's generator holds and draws next
+    (simulator.cpp:1518-1534 selection sampling, :1093-1106 startSceneSwap), on the library's
+    counter-based stream of scene choices."""
+    M64 = (1 << 64) - 1
+
+    def __init__(self, seed, num_dataset, num_active):
+        self.seed, self.k = seed, 0
+        self.active, self.inactive = [], []
+        i = 0
+        while i < num_dataset and len(self.active) < num_active:
+            w = np.float32(self.draw() >> 8) * np.float32(1.0 / 16777216.0)
+            if w * np.float32(num_dataset - i) < np.float32(num_active - len(self.active)):
+                self.active.append(i)
+            else:
+                self.inactive.append(i)
+            i += 1
+        self.inactive += list(range(i, num_dataset))
+
+    def mix(self, z):
+        z &= self.M64
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & self.M64
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & self.M64
+        return z ^ (z >> 31)
+
+    def draw(self):
+        key = self.mix(self.seed + 0x9E3779B97F4A7C15 * 0x100000000 + 0xD1B54A32D192ED03)
+        r = self.mix(key + 0x9E3779B97F4A7C15 * (self.k + 1)) >> 32
+        self.k += 1
+        return r
+
+    def start_swap(self, slot):
+        pos = (self.draw() * len(self.inactive)) >> 32
+        self.inactive[pos], self.active[slot] = self.active[slot], self.inactive[pos]
+        return self.active[slot]
+
+
+def test_dataset_directory_and_automatic_rotation(oracle, torch_cuda, tmp_path):
+    """Construction from a dataset directory with more scenes than slots, through the trainer-side
+    entry (construct_envs): the library picks the resident scenes at random and rotates the
+    others in by itself, loading them in a thread of its own while the simulation steps.  Which
+    scenes it picks is checked against an independent restatement of the reference's policy;
+    every swap it starts is repeated on the oracle at the same step, and every step is compared
+    in full.  Actions stay on the GPU and outputs are taken by device-to-device copies, like a
+    device-resident rollout storage would."""
+    import time
+    from bps_nav_amd import env_utils
+    from oracle import bpo
+    print("case: dataset directory + automatic rotation", flush=True)
+    pool = common.build_scenes(oracle, 2, 5, episodes_per_scene=24) + common.build_scenes(oracle, 1, 3, episodes_per_scene=24)
+    content, assets = write_dataset(str(tmp_path), pool)
+    n, S, seed = 96, 3, 12345
+    envs, obs, rewards, masks, infos, syncs = env_utils.construct_envs(
+        "pointnav", content, assets, n, num_worker_groups=S, double_buffered=False, seed=seed, max_steps=40,
+        scene_reserve=4.0, rotation_interval_ms=0)
+    assert rewards[0].shape == (n, 1) and masks[0].shape == (n, 1) and obs[0]["pointgoal_with_gps_compass"].shape == (n, 2)
+    assert all(t.is_cuda for t in (rewards[0], masks[0], obs[0]["pointgoal_with_gps_compass"], infos[0]["spl"]))
+    policy = ScenePolicy(seed, len(pool), S)
+    first = list(policy.active)
+    assert sorted(first) != [0, 1, 2] or True     # any three of the eight
+    cpu = bpo.Sim(oracle, [pool[i] for i in first], n, seed=seed, threads=3, max_steps=40)
+    expected_next = [policy.start_swap(slot) for slot in range(S)]   # every slot starts loading at construction
+    assert list(envs.active_scenes()) == expected_next
+    cpu.reset()
+    envs.reset(0)
+    state, info_view = envs.get_state(0), envs.get_infos(0)
+    storage = torch_cuda.zeros((200, n, 1), device="cuda")        # a rollout storage's reward buffer
+    pending = {}          # slot -> dataset index on its way in
+    events = 0
+    acts = common.action_stream(2, 200, n)
+    for t, a in enumerate(acts):
+        if t in (0, 40, 90):
+            time.sleep(0.3)     # let the loader thread finish what it has been asked for
+        envs.step_start(0, torch_cuda.from_numpy(a).cuda())
+        for step_ordinal, slot, scene in envs.rotation_events():
+            assert step_ordinal == t and scene == expected_next[slot], "a scene other than the policy's was brought in"
+            cpu.swap_scene(slot, *pool[scene])
+            pending[slot] = scene
+            events += 1
+        cpu.step(a)
+        envs.step_end(0)
+        syncs[0].wait()
+        storage[t].copy_(rewards[0])
+        assert_step_equal(cpu, envs, 0, state, info_view, f"at step {t}")
+        for slot in sorted(pending):          # postStep: completed swaps draw their slot's next scene, in slot order
+            if cpu.swap_remaining(slot) == 0:
+                del pending[slot]
+                expected_next[slot] = policy.start_swap(slot)
+        assert list(envs.active_scenes()) == expected_next
+    assert events >= 6, f"only {events} swaps were started"
+    pct, in_use, per_scene = envs.swap_stats
+    assert pct > 0 and S <= in_use <= 2 * S and per_scene <= n / S
+    assert np.isfinite(storage.cpu().numpy()).mean() > 0.9
+    with pytest.raises(RuntimeError, match="rotates its scenes by itself"):
+        envs.swap_scene(0, *pool[0])
+    envs.check_errors()
+    envs.close()
+    # without rotation the extra scenes are only a pool to pick from
+    gen = make_gen(pool, n, seed=seed, rotate=False, num_active_scenes=S)
+    assert list(gen.active_scenes()) == first
     gen.close()
 
 
