@@ -140,18 +140,9 @@ struct HeapEntry {
 
 // HBM slot of one A* wavefront: the node pool (LDS caches its hot part) and the open-list
 // entries beyond what LDS holds.
-// Log of open-list operations of a search (see geodesic_device.h): one pop and at most six
-// pushes or modifies per expanded node; a search that would outgrow it falls back to the slower
-// exact path, which has not happened in any workload measured (about 6000 entries at most).
-constexpr int kOpLogCap = 16384;
-struct OpLogEntry {
-  uint32_t key;    // total, as bits
-  uint32_t word;   // packed node (node index | polygon index << 11) | operation << 30
-};
 struct alignas(128) GeoSlot {
   ANode nodes[kMaxNodes];
   HeapEntry heap_spill[kMaxNodes];
-  OpLogEntry oplog[kOpLogCap];
 };
 
 struct GeoQuery {
@@ -185,7 +176,7 @@ constexpr uint32_t kCostUnknown = 0xffffffffu;
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,
-  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18, kCntTieRestarts = 19, kCntTieReplays = 20, kCntPrefetchHits = 21   // 8..15: phase cycles of the diagnostic build
+  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18   // 8..15: phase cycles of the diagnostic build
 };
 
 }  // namespace bpsx

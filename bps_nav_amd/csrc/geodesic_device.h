@@ -36,9 +36,6 @@
 
 #ifndef BPSX_GEODESIC_COMMON_H
 #define BPSX_GEODESIC_COMMON_H
-#ifndef BPSX_BAG
-#define BPSX_BAG 1   // 1: searches start with the open list as an unordered set (see OpenBag)
-#endif
 namespace bpsx {
 
 #ifdef BPSX_ASM_MARKS
@@ -220,175 +217,13 @@ struct RegHeap {
   }
 };
 
-// The open list as an unordered set in registers.  dtNodeQueue::pop returns the entry with the
-// smallest total; while that smallest total is held by one entry only, which entry that is does
-// not depend on how the binary heap happens to be arranged, so a set with a minimum search gives
-// the same sequence of pops as the heap, at a fraction of its cost.  Entry p (0-based, dense:
-// entries 0..size-1) lives in lane p & 63 of register pair p >> 6; unused places hold kEmpty
-// keys and kNoNode nodes.  The minimum is found with a cross-lane reduction; push appends,
-// modify rewrites the key of the entry that names the node, pop moves the last entry into the
-// gap.  All writes are lane-predicated vector selects: no branches, no scalar lane writes.
-// When two entries share the smallest total the heap's arrangement decides; the search keeps a
-// log of its open-list operations for that case (see OpLog).
-struct OpenBag {
-  static constexpr int kCap = 128;
-  static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
-  static constexpr uint32_t kNoNode = 0xffffffffu;  // no packed node looks like this (26 bits)
-  uint32_t t0, t1;   // total bits
-  uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11
-  int size;          // places in use: 0..size-1, of which `hole` (if >= 0) is vacant
-  int hole;
-  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = kNoNode; size = 0; hole = -1; }
-  BPSX_DEV int count() const { return size - (hole >= 0 ? 1 : 0); }
-  static BPSX_DEV uint32_t umin(uint32_t v, uint32_t w) { return w < v ? w : v; }
-  // smallest key of the wavefront, as a wave-uniform value
-  static BPSX_DEV uint32_t wave_min(uint32_t v) {
-    // within rows of 16 lanes: exchange over 1, 2, mirror within 8, mirror within 16.  A lane
-    // pattern on an operand needs two idle cycles after the write of that register.
-    asm("s_nop 1\n\t"
-        "v_min_u32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 1\n\t"
-        "v_min_u32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 1\n\t"
-        "v_min_u32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 1\n\t"
-        "v_min_u32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 0"
-        : "+v"(v));
-    // every lane now holds its row's minimum: the four rows meet on the scalar unit
-    const uint32_t a = rlane(v, 0), b = rlane(v, 16), c = rlane(v, 32), d = rlane(v, 48);
-    const uint32_t ab = a < b ? a : b, cd = c < d ? c : d;
-    return ab < cd ? ab : cd;
-  }
-  BPSX_DEV uint32_t key_at(int p) const {
-    const uint32_t a = rlane(t0, p & 63), b = rlane(t1, p & 63);
-    return p < 64 ? a : b;
-  }
-  BPSX_DEV uint32_t node_at(int p) const {
-    const uint32_t a = rlane(n0, p & 63), b = rlane(n1, p & 63);
-    return p < 64 ? a : b;
-  }
-  // Position of the entry with the smallest total and that total; *tie when another entry has
-  // the same total.  The set must not be empty.
-  BPSX_DEV int argmin(bool* tie, uint32_t* key) const {
-    const uint32_t m = wave_min(umin(t0, t1));
-    *key = m;
-    const unsigned long long h0 = __ballot(t0 == m), h1 = __ballot(t1 == m);
-    *tie = __popcll(h0) + __popcll(h1) > 1;
-    return h0 ? __ffsll((long long)h0) - 1 : 64 + __ffsll((long long)h1) - 1;
-  }
-  // position of the entry of node `node` (packed like n0), or -1
-  BPSX_DEV int find(uint32_t node) const {
-    const unsigned long long h0 = __ballot(n0 == node && t0 != kEmpty), h1 = __ballot(n1 == node && t1 != kEmpty);
-    return h0 ? __ffsll((long long)h0) - 1 : (h1 ? 64 + __ffsll((long long)h1) - 1 : -1);
-  }
-  BPSX_DEV void write(int p, uint32_t key, uint32_t node, int lane) {
-    const int hi = lane + 64;
-    t0 = lane == p ? key : t0;
-    n0 = lane == p ? node : n0;
-    t1 = hi == p ? key : t1;
-    n1 = hi == p ? node : n1;
-  }
-  // takes entry p out; its place stays vacant until the next push fills it or settle() closes it
-  BPSX_DEV void take(int p, int lane) {
-    hole = p;
-    t0 = lane == p ? kEmpty : t0;
-    t1 = lane + 64 == p ? kEmpty : t1;
-  }
-  // ---- the set without order of places (astar_spec): an entry may sit anywhere, a vacant place
-  // holds kEmpty; `size` counts the entries
-  // adds an entry at the first vacant place; returns where
-  BPSX_DEV int put(uint32_t key, uint32_t node, int lane) {
-    const unsigned long long v0 = __ballot(t0 == kEmpty);
-    int p;
-    if (v0) p = __ffsll((long long)v0) - 1;
-    else p = 64 + __ffsll((long long)__ballot(t1 == kEmpty)) - 1;
-    size++;
-    write(p, key, node, lane);
-    return p;
-  }
-  // takes the entry at place p out
-  BPSX_DEV void drop(int p, int lane) {
-    size--;
-    t0 = lane == p ? kEmpty : t0;
-    t1 = lane + 64 == p ? kEmpty : t1;
-  }
-  // adds an entry; returns where
-  BPSX_DEV int push(uint32_t key, uint32_t node, int lane) {
-    int p;
-    if (hole >= 0) { p = hole; hole = -1; }
-    else { p = size; size = p + 1; }
-    write(p, key, node, lane);
-    return p;
-  }
-  // Closes a vacant place left at the end of an expansion: the last entry moves into it.
-  // Returns the position the last entry had if it moved (so that the caller can follow it), else -1.
-  BPSX_DEV int settle(int lane, int* to) {
-    if (hole < 0) return -1;
-    const int h = hole, last = size - 1;
-    *to = h;
-    hole = -1;
-    size = last;
-    if (h == last) return -1;   // the vacant place was the last one: its key is kEmpty already
-    const uint32_t lt = key_at(last), ln = node_at(last);
-    write(h, lt, ln, lane);
-    t0 = lane == last ? kEmpty : t0;
-    t1 = lane + 64 == last ? kEmpty : t1;
-    return last;
-  }
-  // the entry of node `node` gets key `key`
-  BPSX_DEV void modify(uint32_t node, uint32_t key) {
-    t0 = (n0 == node && t0 != kEmpty) ? key : t0;
-    t1 = (n1 == node && t1 != kEmpty) ? key : t1;
-  }
-};
-
-// Log of a search's open-list operations, in the wavefront's HBM slot: what is needed to
-// rebuild the reference's binary heap at the moment two open entries share the smallest total.
-// Replaying the log through the exact heap (RegHeap) gives the heap's arrangement and with it
-// the entry dtNodeQueue::pop would return; the search then carries on with the set, and the
-// next tie replays only what was logged since.  word = packed node | op << 30.
-constexpr uint32_t kOpPush = 0u, kOpModify = 1u, kOpPop = 2u;
-
 struct AstarState {
   int lastBest;
   float lastBestCost;
   bool outOfNodes;
   RegHeap rh;
-  OpenBag bag;
-  int logPos;      // entries written to the operation log
-  int logDone;     // entries of it already applied to rh
-  // the entry that will be popped next: position, key and how many entries hold that key
-  int nextPos, nextCount;
-  uint32_t nextKey, nextNode;
-  AEdge pf;        // edge records of polygon pfIp, requested ahead (lanes 0..5)
-  uint32_t pfIp;
-  // ---- two-at-a-time expansion (astar_spec): the smallest open entries wait in four slots,
-  // slot s in lanes 8 s .. 8 s + 5, with their polygons' edge records already requested
-  uint32_t fKey, fNode;     // per lane: key and packed node of the lane's slot (kEmpty: slot vacant)
-  AEdge fe;                 // per lane: edge record (lane & 7) of the slot's polygon
-  uint32_t bmKey, bmNode;   // smallest entry of the set (the open entries not in a slot) ...
-  int bmPos, bmCount;       // ... its place, and how many entries hold that key (0: set empty)
-  uint32_t forceNode;       // after a tie was resolved from the log: the node to expand next (kNoNode: none)
 };
-constexpr int kSlots = 4;
 enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
-
-// Applies entries [from, to) of the operation log to the exact heap.
-BPSX_DEV void replay_log(RegHeap& rh, const OpLogEntry* log, int from, int to, int lane) {
-  for (int base = from; base < to; base += 64) {
-    OpLogEntry e{0u, 0u};
-    if (base + lane < to) e = log[base + lane];
-    const int n = to - base < 64 ? to - base : 64;
-    for (int i = 0; i < n; ++i) {
-      const uint32_t key = rlane(e.key, i), w = rlane(e.word, i);
-      const uint32_t op = w >> 30, node = w & 0x3fffffffu;
-      if (op == kOpPop) rh.pop(lane);
-      else if (op == kOpPush) rh.push(key, node, lane);
-      else rh.modify(node, key, lane);
-    }
-  }
-}
 
 BPSX_DEV float tri_area2d(const float* a, const float* b, const float* c) {
   const float abx = b[0] - a[0], abz = b[2] - a[2];
@@ -463,9 +298,6 @@ struct GeoWave {
   int heapSize;
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
-  uint32_t tieRestarts;              // queries run again with the exact heap (open list or log outgrew the fast path)
-  uint32_t tieReplays;               // ties resolved by replaying the operation log
-  uint32_t prefetchHits;             // expansions whose edge records had been requested ahead
 #ifdef BPSX_QUERY_TRACE
   uint32_t missTop, missNb, maxHeap;
 #endif
@@ -587,12 +419,9 @@ struct GeoWave {
   }
 };
 
-// The expansion loop of findPath.  M = 3: open list as an unordered set in registers, all links
-// in LDS; M = 4: the same, links may spill.  These two return kAstarTie when two open entries
-// share the smallest total; the search then starts again with the exact heap: M = 0: heap in
-// registers, all links in LDS; M = 1: heap in registers, links may spill; M = 2: heap in
-// LDS/HBM, links may spill.  Returns kAstarGrow* before an expansion that could outgrow what
-// its mode holds.
+// The expansion loop of findPath.  M = 0: open list in registers, all links in LDS; M = 1: open
+// list in registers, links may spill; M = 2: open list in LDS/HBM, links may spill.  Returns
+// kAstarGrow* before an expansion that could outgrow what its mode holds.
 template <int M>
 BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
 #ifdef BPSX_PHASE_TIMING
@@ -604,43 +433,17 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const float H_SCALE = 0.999f;
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
   endIp = (uint32_t)uniform_i((int)endIp);   // the same in all lanes: the goal test stays on the scalar unit
-  constexpr bool S = M == 1 || M == 2 || M == 4;    // links and states may be in HBM
+  constexpr bool S = M >= 1;    // links and states may be in HBM
   constexpr bool SH = M == 2;   // open list in LDS/HBM
-  constexpr bool BAG = M >= 3;  // open list as an unordered set
   RegHeap& rh = st.rh;
-  OpenBag& bag = st.bag;
-  while ((SH ? g.heapSize : (BAG ? bag.size : rh.size)) > 0) {   // (the set has no vacant place here: size is its count)
-    if (!S && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
-    if (!SH && !BAG && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
-    // the set, the heap that is rebuilt from the log on a tie, and the log itself must hold one more expansion
-    if (BAG && (bag.size > kRegHeap - kNvp || st.logPos > kOpLogCap - 2 * kNvp)) return kAstarGrowHeap;
-    // the node about to be popped is known before the open list is repaired: fetch its edges
-    // meanwhile
+  while ((SH ? g.heapSize : rh.size) > 0) {
+    if (M == 0 && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
+    if (!SH && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
+    // the node about to be popped is the root: fetch its edges while the heap is repaired
     int bi;
     uint32_t bestIp;
     uint32_t blink;   // the node's link word: closing the node rewrites its flags
-    int bagPos = 0;
-    if (BAG) {
-      // The smallest entry is known from the end of the previous expansion: the runner-up found
-      // then, unless a key written since is smaller (st.next*).
-      bagPos = st.nextPos;
-      uint32_t root;
-      if (st.nextCount > 1) {
-        // two open entries share the smallest total: the reference's heap decides.  Bring the
-        // exact heap up to date from the log; its root is the entry to pop.
-        wave_sync();
-        replay_log(rh, g.ws->oplog, st.logDone, st.logPos, lane);
-        st.logDone = st.logPos;
-        g.tieReplays++;
-        root = rlane(rh.n0, 1);
-        bagPos = bag.find(root);
-      } else {
-        root = st.nextNode;
-      }
-      bi = (int)(root & 0x7ffu);
-      bestIp = root >> 11;
-      blink = g.link<S>(bi);
-    } else if (SH) {
+    if (SH) {
       bi = uniform_i((int)L->heap[0].node);
       blink = g.link<S>(bi);
       bestIp = link_id((uint32_t)uniform_i((int)blink));
@@ -652,13 +455,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
-    // its edge records were requested one expansion ago if it was the runner-up then
-    const bool prefetched = BAG && bestIp == st.pfIp;
-    if (prefetched) {
-      nb = st.pf.nb; m0 = st.pf.mid[0]; m1 = st.pf.mid[1]; m2 = st.pf.mid[2];
-      if (lane >= kNvp) nb = kNoNb;
-      g.prefetchHits++;
-    } else if (lane < kNvp) {
+    if (lane < kNvp) {
       const AEdge e = edges[bestIp * kNvp + lane];
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
@@ -683,22 +480,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (!SH && (uint32_t)rh.size > g.maxHeap) g.maxHeap = (uint32_t)rh.size;
 #endif
     PHASE_MARK(0);
-    if (BAG) {
-      bag.take(bagPos, lane);
-      // the smallest of what remains is the next node to expand unless this expansion writes a
-      // smaller key: note it, and request its polygon's edge records now
-      st.nextCount = 0;
-      st.pfIp = kNoNb;
-      if (bag.size > 1) {
-        bool tie;
-        st.nextPos = bag.argmin(&tie, &st.nextKey);
-        st.nextCount = tie ? 2 : 1;
-        st.nextNode = bag.node_at(st.nextPos);
-        st.pfIp = st.nextNode >> 11;
-        if (lane < kNvp) st.pf = edges[st.pfIp * kNvp + lane];
-      }
-    }
-    else if (SH) g.pop<true>();
+    if (SH) g.pop<true>();
     else rh.pop(lane);
     const uint32_t pidx = (uint32_t)uniform_i((int)bparent);
     PHASE_MARK(1);
@@ -814,36 +596,13 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     // then the open list
     unsigned long long upd = __ballot(update);
     const unsigned long long openMask = __ballot(wasOpen);
-    if (BAG) {
-      // log: this expansion's pop (written by lane 63, which handles no edge), then its updates in edge order
-      const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(upd >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)upd, 0u));
-      if (update || lane == 63) {
-        OpLogEntry e;
-        e.key = __float_as_uint(total);
-        e.word = update ? (packed | ((wasOpen ? kOpModify : kOpPush) << 30)) : (kOpPop << 30);
-        g.ws->oplog[st.logPos + (update ? 1 + rank : 0)] = e;
-      }
-      st.logPos += 1 + __popcll(upd);
-    }
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
       const uint32_t entry = rlane(packed, src);
       const float t = lane_f(total, src);
       const bool open = (openMask >> src) & 1ull;
-      if (BAG) {
-        const uint32_t key = __float_as_uint(t);
-        int at;
-        if (open) { at = bag.find(entry); bag.modify(entry, key); }
-        else at = bag.push(key, entry, lane);
-        if (st.nextCount != 0 && at == st.nextPos) {
-          st.nextKey = key; st.nextCount = 1;   // the smallest entry itself got a smaller key
-        } else if (key < st.nextKey || st.nextCount == 0) {
-          st.nextKey = key; st.nextPos = at; st.nextCount = 1; st.nextNode = entry;
-        } else if (key == st.nextKey) {
-          st.nextCount++;
-        }
-      } else if (SH) {
+      if (SH) {
         if (open) g.modify<true>((int)(entry & 0x7ffu), t);
         else g.push<true>(t, (int)(entry & 0x7ffu));
       } else {
@@ -851,390 +610,9 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         else rh.push(__float_as_uint(t), entry, lane);
       }
     }
-    if (BAG) {
-      // no push took the popped entry's place: close it, and follow the smallest entry if it is the one that moves
-      int to = 0;
-      const int moved = bag.settle(lane, &to);
-      if (moved >= 0 && st.nextCount != 0 && st.nextPos == moved) st.nextPos = to;
-    }
     PHASE_MARK(6);
   }
   return kAstarEmpty;
-}
-
-// The expansion loop of findPath, two nodes at a time.
-//
-// The reference expands one node per iteration: the open node with the smallest total.  Here the
-// two smallest (A, then B) are worked on by the same instructions in different lanes: edge
-// records, node lookup and costs of both are computed together, without side effects, from the
-// state before either expansion.  A's results are then committed.  B's results are what the
-// reference would compute after A's expansion, and are committed too, if
-//   - B is still the node the reference would pop next: none of A's updates has a total at or
-//     below B's, and no other open entry shares B's total,
-//   - nothing B looked at was changed by A: B evaluates no polygon that A evaluates, not A's own
-//     polygon, and A does not evaluate B's polygon,
-//   - B is not the goal, and the node pool has room for both.
-// Otherwise B simply stays where it is and is A in the next iteration.  On the benchmark's
-// scenes three iterations out of four commit both, which nearly halves the instructions per
-// expanded node: a search is one chain of dependent instructions, and its length, not memory
-// bandwidth, sets the time of the longest searches and of the launch.
-//
-// The open entries live in a register set (OpenBag); the smallest ones are moved ahead of time
-// into four slots (lanes 8 s .. 8 s + 5) whose polygons' edge records are requested at once, so
-// that they have arrived when the slot's turn comes.  Ties for the smallest total are resolved
-// by replaying the operation log through the exact heap, as the order then depends on the
-// heap's arrangement.  S: node links may be in HBM (more than kLinksLds nodes).
-template <bool S>
-BPSX_DEV AstarExit astar_spec(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
-#ifdef BPSX_PHASE_TIMING
-                              , unsigned long long* phase_acc, unsigned long long& phase_t0
-#endif
-                              ) {
-  const int lane = g.lane;
-  GeoLds* L = g.L;
-  const float H_SCALE = 0.999f;
-  const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
-  endIp = (uint32_t)uniform_i((int)endIp);
-  const int slot = lane >> 3, el = lane & 7;
-  const bool edgeLane = slot < kSlots && el < kNvp;
-  OpenBag& bag = st.bag;
-  RegHeap& rh = st.rh;
-  constexpr uint32_t kE = OpenBag::kEmpty;
-
-  // the set's smallest entry, after its contents changed in ways the running record does not follow
-  auto rescan = [&]() {
-    st.bmCount = 0;
-    if (bag.size > 0) {
-      bool tie;
-      st.bmPos = bag.argmin(&tie, &st.bmKey);
-      st.bmCount = tie ? 2 : 1;
-      st.bmNode = bag.node_at(st.bmPos);
-    }
-  };
-  // an entry enters the set: keep the record of the smallest
-  auto bag_push = [&](uint32_t key, uint32_t node) {
-    const int at = bag.put(key, node, lane);
-    if (st.bmCount == 0 || key < st.bmKey) { st.bmKey = key; st.bmPos = at; st.bmNode = node; st.bmCount = 1; }
-    else if (key == st.bmKey) st.bmCount++;
-  };
-  // the set's entry at `pos` moves into slot s, and its polygon's edge records are requested
-  auto bring = [&](int pos, uint32_t key, uint32_t node, int s) {
-    bag.drop(pos, lane);
-    if (slot == s) { st.fKey = key; st.fNode = node; }
-    if (slot == s && el < kNvp) st.fe = edges[(node >> 11) * kNvp + (uint32_t)el];
-    rescan();
-  };
-
-  // Every pass either expands a node or moves an entry into a slot; a search expands a few thousand
-  // nodes at most.  The bound only guards against an endless loop should the bookkeeping ever
-  // be inconsistent: the caller then runs the search again on the plain path.
-  for (int pass = 0;; ++pass) {
-    if (pass > 16 * kMaxNodes) return kAstarGrowHeap;
-    // room for two more expansions in whatever is bounded
-    if (!S && g.nodeCount > kLinksLds - 2 * kNvp) return kAstarGrowLinks;
-    if (bag.size + kSlots > kRegHeap - 2 * kNvp || st.logPos > kOpLogCap - 4 * kNvp) return kAstarGrowHeap;
-    // ---- the slots' keys, and the smallest three of them (a tournament of four)
-    const uint32_t k0 = rlane(st.fKey, 0), k1 = rlane(st.fKey, 8), k2 = rlane(st.fKey, 16), k3 = rlane(st.fKey, 24);
-    uint32_t ka, kb, kc;
-    int sa, sb;
-    {
-      const bool c01 = k1 < k0, c23 = k3 < k2;
-      const uint32_t a01 = c01 ? k1 : k0, b01 = c01 ? k0 : k1, a23 = c23 ? k3 : k2, b23 = c23 ? k2 : k3;
-      const int i01 = c01 ? 1 : 0, j01 = c01 ? 0 : 1, i23 = c23 ? 3 : 2, j23 = c23 ? 2 : 3;
-      const bool cf = a23 < a01;
-      ka = cf ? a23 : a01; sa = cf ? i23 : i01;
-      const uint32_t lf = cf ? a01 : a23, ls = cf ? b23 : b01;     // the final's loser, the winner's semi-final loser
-      const int ilf = cf ? i01 : i23, ils = cf ? j23 : j01;
-      const bool cs = ls < lf;
-      kb = cs ? ls : lf; sb = cs ? ils : ilf;
-      const uint32_t r1 = cs ? lf : ls, r2 = cf ? b01 : b23;
-      kc = r2 < r1 ? r2 : r1;
-    }
-    const bool bagHas = st.bmCount > 0;
-    if (ka == kE && !bagHas) return kAstarEmpty;   // nothing open any more
-    if (st.forceNode == OpenBag::kNoNode) {
-      // the smallest open entry must be in a slot: it may be in the set instead (an entry written
-      // by the last expansion, or the slots have just been emptied)
-      if (bagHas && (ka == kE || st.bmKey < ka)) {
-        if (st.bmCount > 1) {
-          // ... and shares its total with another entry of the set: the heap decides (below)
-          ka = st.bmKey;
-        } else {
-          int s = k0 == kE ? 0 : (k1 == kE ? 1 : (k2 == kE ? 2 : (k3 == kE ? 3 : -1)));
-          if (s < 0) {
-            // every slot is taken: the one with the largest total goes back to the set
-            uint32_t kw = k0; s = 0;
-            if (k1 > kw) { kw = k1; s = 1; }
-            if (k2 > kw) { kw = k2; s = 2; }
-            if (k3 > kw) { kw = k3; s = 3; }
-            const int keep = st.bmPos;      // places do not move when an entry is added
-            const uint32_t kk = st.bmKey, kn = st.bmNode;
-            bag_push(kw, rlane(st.fNode, s * 8));
-            bring(keep, kk, kn, s);
-          } else {
-            bring(st.bmPos, st.bmKey, st.bmNode, s);
-          }
-          continue;
-        }
-      }
-      // is the smallest total held by one entry only?
-      const bool tie = kb == ka || (bagHas && st.bmKey == ka);
-      if (tie) {
-        // The reference's heap decides.  Bring the exact heap up to date from the log; its
-        // root is the entry to pop.
-        wave_sync();
-        replay_log(rh, g.ws->oplog, st.logDone, st.logPos, lane);
-        st.logDone = st.logPos;
-        g.tieReplays++;
-        st.forceNode = rlane(rh.n0, 1);
-        continue;
-      }
-    } else {
-      // the node the exact heap named: in a slot, or to be moved to one
-      const uint32_t want = st.forceNode;
-      const uint32_t n0 = rlane(st.fNode, 0), n1 = rlane(st.fNode, 8), n2 = rlane(st.fNode, 16), n3 = rlane(st.fNode, 24);
-      sa = (k0 != kE && n0 == want) ? 0 : ((k1 != kE && n1 == want) ? 1 : ((k2 != kE && n2 == want) ? 2 : ((k3 != kE && n3 == want) ? 3 : -1)));
-      if (sa < 0) {
-        int s = k0 == kE ? 0 : (k1 == kE ? 1 : (k2 == kE ? 2 : (k3 == kE ? 3 : -1)));
-        const int pos = bag.find(want);
-        if (pos < 0) return kAstarGrowHeap;   // cannot happen: the heap's root is an open entry
-        if (s < 0) {
-          uint32_t kw = k0; s = 0;
-          if (k1 > kw) { kw = k1; s = 1; }
-          if (k2 > kw) { kw = k2; s = 2; }
-          if (k3 > kw) { kw = k3; s = 3; }
-          bag_push(kw, rlane(st.fNode, s * 8));
-        }
-        bring(pos, bag.key_at(pos), want, s);
-        continue;
-      }
-      ka = rlane(st.fKey, sa * 8);
-    }
-    const bool forced = st.forceNode != OpenBag::kNoNode;
-    st.forceNode = OpenBag::kNoNode;
-    // ---- A is slot sa.  B: the smallest of the other slots, if it is the second smallest open entry.
-    const uint32_t nodeA = rlane(st.fNode, sa * 8);
-    const int biA = (int)(nodeA & 0x7ffu);
-    const uint32_t ipA = nodeA >> 11;
-    if (forced) {
-      // (the forced slot need not hold the smallest key of the slots' tournament: find the runner-up anew)
-      kb = kE; sb = 0; kc = kE;
-    }
-    const uint32_t nodeB = rlane(st.fNode, sb * 8);
-    const uint32_t ipB = nodeB >> 11;
-    if (ipA == endIp) {
-      // the goal is popped: closed, not expanded
-      if (lane == 0) g.set_link<S>(biA, with_flags(g.link<S>(biA), 2u));
-      st.lastBest = biA;
-      return kAstarGoal;
-    }
-    const bool spec = !forced && kb != kE && kc != kb && kb > ka && (!bagHas || kb < st.bmKey) && ipB != endIp &&
-                      (!S || g.nodeCount + 2 * kNvp <= kMaxNodes);
-    PHASE_MARK(0);
-    // ---- slots vacated by the last pass take the set's smallest entries now: their polygons'
-    // edge records are on the way while this pass works on A and B (whose records are taken
-    // out of the slot registers first, so that nothing below waits for the new requests)
-    const AEdge cur = st.fe;
-    const uint32_t curNode = st.fNode;
-    if (st.bmCount > 0 && k0 == kE) bring(st.bmPos, st.bmKey, st.bmNode, 0);
-    if (st.bmCount > 0 && k1 == kE) bring(st.bmPos, st.bmKey, st.bmNode, 1);
-    if (st.bmCount > 0 && k2 == kE) bring(st.bmPos, st.bmKey, st.bmNode, 2);
-    if (st.bmCount > 0 && k3 == kE) bring(st.bmPos, st.bmKey, st.bmNode, 3);
-    PHASE_MARK(1);
-    // ---- both expansions, lane-wise, without side effects
-    const bool inA = slot == sa, inB = spec && slot == sb;
-    const bool act = edgeLane && (inA || inB);
-    const int bi = (int)(curNode & 0x7ffu);       // the lane's slot's node
-    uint32_t nb = act ? cur.nb : kNoNb;
-    const float m0 = cur.mid[0], m1 = cur.mid[1], m2 = cur.mid[2];
-    // the expanded nodes' own position, cost and parent
-    float b0, b1, b2, bcost;
-    uint32_t pidx;
-    {
-      const int bis = act ? bi : 0;
-      const int w = bis & (kWindow - 1);
-      b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
-      pidx = L->w_parent[w];
-      const bool gone = act && !g.in_window(bis);
-      if (__ballot(gone)) {
-        if (gone) {
-          BPSX_KEEP_APART();
-          const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bis].pos);   // pos, cost
-          b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
-          pidx = g.ws->nodes[bis].parent;
-          BPSX_KEEP_APART();
-        }
-      }
-    }
-    const uint32_t bucket = GeoWave::hash(nb);
-    uint32_t chainHead, hitLink;
-    int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
-    // the polygon the expanded node was reached from is not entered again
-    if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
-    PHASE_MARK(2);
-    const bool valid = nb != kNoNb;
-    const bool isNew = valid && ni < 0;
-    float p0, p1, p2, oldTotal;
-    uint32_t fl = link_flags(hitLink);
-    {
-      const int nis = (valid && !isNew) ? ni : 0;
-      const int w = nis & (kWindow - 1);
-      p0 = L->w_pos[0][w]; p1 = L->w_pos[1][w]; p2 = L->w_pos[2][w]; oldTotal = L->w_total[w];
-      const bool miss = valid && !isNew && !g.in_window(nis);
-      if (__ballot(miss)) {
-        if (miss) {
-          BPSX_KEEP_APART();
-          const ANode& hn = g.ws->nodes[nis];
-          const float4 pc = *reinterpret_cast<const float4*>(hn.pos);
-          p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = hn.total;
-          BPSX_KEEP_APART();
-        }
-      }
-    }
-    if (isNew) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }
-    const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
-    const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
-    const float curCost = sqrt_exact(cx * cx + cy * cy + cz * cz) * 1.0f;
-    const float toEnd = sqrt_exact(ex * ex + ey * ey + ez * ez);
-    const bool last = nb == endIp;
-    const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
-    const float heuristic = last ? 0.0f : toEnd * H_SCALE;
-    const float total = cost + heuristic;
-    const bool update = valid && !(fl && total >= oldTotal);
-    const bool wasOpen = update && (fl & 1u) != 0;
-    PHASE_MARK(3);
-    // ---- may B be committed after A?
-    bool commitB = spec;
-    if (spec) {
-      // A's new totals all lie above B's, so that B stays the next to pop
-      if (__ballot(inA && update && __float_as_uint(total) <= kb)) commitB = false;
-      // B evaluates A's polygon, or A evaluates B's
-      if (__ballot((inB && nb == ipA) || (inA && nb == ipB))) commitB = false;
-      // a polygon both evaluate
-      unsigned long long both = 0;
-#pragma unroll
-      for (int j = 0; j < kNvp; ++j) {
-        const uint32_t aj = rlane(nb, sa * 8 + j);
-        both |= __ballot(inB && nb == aj && aj != kNoNb);
-      }
-      if (both) commitB = false;
-    }
-    PHASE_MARK(4);
-    // ---- commit: A's results, and B's behind them
-    if (commitB) g.prefetchHits++;
-    const bool mine = inA || (commitB && inB);
-    const unsigned long long mA = 0x3full << (sa * 8), mB = commitB ? 0x3full << (sb * 8) : 0ull;
-    *pops += commitB ? 2u : 1u;
-    if (lane == sa * 8 || (commitB && lane == sb * 8)) g.set_link<S>(bi, with_flags(g.link<S>(bi), 2u));   // open -> closed
-    // new nodes take consecutive indices in edge order, A's before B's; past the pool's end the search stops
-    const bool newM = mine && isNew;
-    const unsigned long long need = __ballot(newM);
-    if (need) {
-      const unsigned long long needA = need & mA, needB = need & mB;
-      const int cntA = __popcll(needA), count = __popcll(need);
-      const int rank = inA ? (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(needA >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)needA, 0u))
-                           : cntA + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(needB >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)needB, 0u));
-      const int want = g.nodeCount + count;
-      // the reference carries on without the dropped nodes, but reports anything found after
-      // that as failure (only plain DT_SUCCESS counts, PathFinder.cpp:506): the search can stop
-      if (S && want > kMaxNodes) { st.outOfNodes = true; return kAstarEmpty; }
-      if (newM) ni = g.nodeCount + rank;
-      g.nodeCount = want;
-      // All insert at once in front of the chain head their lookup saw (the state before either
-      // expansion).  Of several that share a bucket one store wins; the others see that when
-      // they read the head back and go round again behind the winner.
-      uint32_t head = chainHead;
-      bool pending = newM;
-      for (;;) {
-        if (pending) {
-          g.set_link<S>(ni, make_link(nb, 1u, head));
-          L->first[bucket] = (uint16_t)ni;
-        }
-        wave_sync();
-        if (count == 1) break;
-        if (pending) {
-          head = L->first[bucket];
-          pending = head != (uint32_t)ni;
-        }
-        wave_sync();
-        if (!__ballot(pending)) break;
-      }
-    }
-    const bool upd = mine && update;
-    if (upd) {
-      if (!isNew) g.set_link<S>(ni, with_flags(hitLink, 1u));   // open (again)
-      const int w = ni & (kWindow - 1);
-      if (g.in_window(ni)) {     // with the pool as it is now: an old node may just have left the window
-        L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2;
-        L->w_cost[w] = cost; L->w_total[w] = total;
-        L->w_parent[w] = (uint16_t)(bi + 1);
-      }
-      ANode& hn = g.ws->nodes[ni];
-      *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
-      *reinterpret_cast<uint2*>(&hn.total) = make_uint2(__float_as_uint(total), (uint32_t)(bi + 1));
-    }
-    wave_sync();
-    PHASE_MARK(5);
-    // the "nearest so far" record (lastBestNode of findPath): A's updates in edge order, then B's
-    const uint32_t packed = (uint32_t)ni | (nb << 11);
-    {
-      const unsigned long long better = __ballot(upd && heuristic < st.lastBestCost);
-      if (better) {
-        unsigned long long part[2] = {better & mA, better & mB};
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-          while (part[t]) {
-            const int src = __ffsll((long long)part[t]) - 1;
-            part[t] &= part[t] - 1;
-            const float h = lane_f(heuristic, src);
-            if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
-          }
-      }
-    }
-    // log: A's pop (written by lane 63, which handles no edge), A's updates in edge order, then
-    // B's pop (lane 62) and updates
-    unsigned long long um = __ballot(upd);
-    const unsigned long long openMask = __ballot(upd && wasOpen);
-    {
-      const unsigned long long umA = um & mA, umB = um & mB;
-      const int cuA = __popcll(umA);
-      const int at = inA ? 1 + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(umA >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)umA, 0u))
-                         : 2 + cuA + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(umB >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)umB, 0u));
-      if (upd || lane == 63 || (commitB && lane == 62)) {
-        OpLogEntry e;
-        e.key = __float_as_uint(total);
-        e.word = upd ? (packed | ((wasOpen ? kOpModify : kOpPush) << 30)) : (kOpPop << 30);
-        g.ws->oplog[st.logPos + (upd ? at : (lane == 63 ? 0 : 1 + cuA))] = e;
-      }
-      st.logPos += (commitB ? 2 : 1) + __popcll(um);
-    }
-    PHASE_MARK(6);
-    // the expanded nodes' slots are vacant now
-    if (mine) st.fKey = kE;
-    // the open entries: a node already open is in a slot or in the set
-    while (um) {
-      const int src = __ffsll((long long)um) - 1;
-      um &= um - 1;
-      const uint32_t entry = rlane(packed, src);
-      const uint32_t key = __float_as_uint(lane_f(total, src));
-      if ((openMask >> src) & 1ull) {
-        // in a slot?  (a slot just vacated keeps its old node: that one is closed, and a closed node is pushed, not modified)
-        const unsigned long long inSlot = __ballot(st.fNode == entry && st.fKey != kE);
-        if (inSlot) {
-          if (st.fNode == entry && st.fKey != kE) st.fKey = key;
-        } else {
-          const int at = bag.find(entry);
-          if (at < 0) return kAstarGrowHeap;   // cannot happen: an open node is in a slot or in the set
-          bag.modify(entry, key);
-          if (at == st.bmPos) { st.bmKey = key; st.bmCount = 1; }
-          else if (key < st.bmKey) { st.bmKey = key; st.bmPos = at; st.bmNode = entry; st.bmCount = 1; }
-          else if (key == st.bmKey) st.bmCount++;
-        }
-      } else {
-        bag_push(key, entry);
-      }
-    }
-  }
 }
 
 // Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
@@ -1261,9 +639,8 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #else
 #define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
 #endif
-  float startTotal;
-  auto begin = [&]() {
-    g.clear();
+  g.clear();
+  {
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
     const float total = sqrtf(dx * dx + dy * dy + dz * dz) * 0.999f;
     g.nodeCount = 1;
@@ -1282,44 +659,11 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.lastBest = 0;
     st.lastBestCost = total;
     st.outOfNodes = false;
-    startTotal = total;
-  };
-  AstarExit ex;
-#if BPSX_BAG
-  begin();
-  st.bag.init();
-  st.rh.init();
-  if (lane == 0) g.ws->oplog[0] = OpLogEntry{__float_as_uint(startTotal), (startIp << 11) | (kOpPush << 30)};
-  st.logPos = 1;
-  st.logDone = 0;
-  st.bmCount = 0; st.bmPos = 0; st.bmKey = OpenBag::kEmpty; st.bmNode = OpenBag::kNoNode;
-  st.forceNode = OpenBag::kNoNode;
-  // the start node waits in slot 0
-  st.fKey = (lane >> 3) == 0 ? __float_as_uint(startTotal) : OpenBag::kEmpty;
-  st.fNode = (lane >> 3) == 0 ? startIp << 11 : OpenBag::kNoNode;
-  st.fe = AEdge{{0.f, 0.f, 0.f}, kNoNb};
-  if (lane < kNvp) st.fe = edges[startIp * kNvp + (uint32_t)lane];
-#ifdef BPSX_PHASE_TIMING
-#define ASTAR_SPEC(S) astar_spec<S>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0)
-#else
-#define ASTAR_SPEC(S) astar_spec<S>(g, st, edges, endIp, endPos, pops)
-#endif
-  ex = ASTAR_SPEC(false);
-  if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_SPEC(true); }
-#undef ASTAR_SPEC
-#else
-  ex = kAstarGrowHeap;
-#endif
-  if (ex == kAstarGrowHeap) {
-    // the open list has outgrown the register set (or the log its space): the search is done
-    // again with the heap itself, which can spill
-    if (BPSX_BAG) g.tieRestarts++;
-    begin();
     st.rh.init();
-    st.rh.push(__float_as_uint(startTotal), startIp << 11, lane);
-    ex = ASTAR_RUN(0);
-    if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
+    st.rh.push(__float_as_uint(total), startIp << 11, lane);
   }
+  AstarExit ex = ASTAR_RUN(0);
+  if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
   if (ex == kAstarGrowHeap) {
     g.heapSpills++;
     // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap

@@ -175,14 +175,8 @@ int bpsx_check_errors(bpsx_sim *sim);
  * more node links than the kernel keeps in LDS, [17] path searches whose open list outgrew
  * the kernel's registers (both continue in slower code; results are the same), [18] path
  * searches expected to be among the longest of their step, which the kernel runs with larger
- * LDS structures (same results), [19] path searches whose open list outgrew the kernel's fast
- * register set and which were run again with the reference's binary heap (same results),
- * [20] times two open nodes shared the smallest total, so that the arrangement of the
- * reference's binary heap decided which is expanded first: the kernel then rebuilds that heap
- * from its log of the search's open-list operations (same results), [21] node expansions
- * whose polygon's edge records had been requested ahead, while the polygon it was reached
- * from was expanded. */
-#define BPSX_NUM_COUNTERS 22
+ * LDS structures (same results). */
+#define BPSX_NUM_COUNTERS 19
 int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
 /* Per-kernel timing with HIP events on the step's own stream. While enabled, every
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
