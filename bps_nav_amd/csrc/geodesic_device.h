@@ -91,7 +91,7 @@ BPSX_DEV float lanes_down8(float v) {
 // between takes the library routine.
 BPSX_DEV float sqrt_exact(float x) {
   const uint32_t xb = __float_as_uint(x);
-  if (__ballot(xb - 1u < 0x0f800000u - 1u)) return sqrtf(x);   // 0 < x < 2^-96 in some lane: never in practice
+  if (__builtin_expect(__ballot(xb - 1u < 0x0f800000u - 1u) != 0, 0)) return sqrtf(x);   // 0 < x < 2^-96 in some lane: never in practice
   const float s = __builtin_amdgcn_sqrtf(x);
   const float down = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
   const float rdown = fmaf(-down, s, x), rup = fmaf(-up, s, x);
@@ -122,8 +122,26 @@ struct RegHeap {
   uint32_t n0, n1;   // node index (bits 0-10) | the node's polygon index << 11, so that popping
                      // the root names the edge records to fetch without a detour through LDS
   int size;
+  // constants of the lane: the positions that must each be the smaller of their sibling pair
+  // for the hole of a pop to pass through position `lane` (itself and its ancestors below the
+  // root), as a bit set, and the same for the parent of position 64 + lane
+  uint32_t anc0, anc1, panc0, panc1;
   static constexpr uint32_t kEmpty = 0x7fffffffu;   // above +inf; every key stays below 2^31
-  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = 0; size = 0; }
+  static BPSX_DEV unsigned long long route_set(int q) {
+    unsigned long long m = 0;
+    for (; q >= 2; q >>= 1) m |= 1ull << q;
+    return m;
+  }
+  BPSX_DEV void init(int lane) {
+    t0 = t1 = kEmpty; n0 = n1 = 0; size = 0;
+    const unsigned long long a = route_set(lane), pa = route_set(32 + (lane >> 1));
+    anc0 = (uint32_t)a; anc1 = (uint32_t)(a >> 32);
+    panc0 = (uint32_t)pa; panc1 = (uint32_t)(pa >> 32);
+  }
+  // v of the neighbouring lane (lane ^ 1)
+  static BPSX_DEV uint32_t quad_swap(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xb1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, false);
+  }
   static BPSX_DEV uint32_t xlane(int src_lane, uint32_t v) {   // v of another lane; all lanes must be active
     return (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane * 4, (int)v);
   }
@@ -149,27 +167,67 @@ struct RegHeap {
     t0 = parentMoves ? pk : (land ? t : t0);
     n0 = parentMoves ? pn : (land ? n : n0);
   }
+  // The same walk on the scalar unit: q, t and n are wave-uniform, the parents' keys are read
+  // with lane reads, and an entry of A* mostly stays where it is put or moves a level or two.
+  BPSX_DEV void put(int q, uint32_t t, uint32_t n) {
+    if (q < 64) { t0 = wlane(t0, t, q); n0 = wlane(n0, n, q); }
+    else { t1 = wlane(t1, t, q & 63); n1 = wlane(n1, n, q & 63); }
+  }
+  BPSX_DEV void sift_up(int q, uint32_t t, uint32_t n) {
+    while (q > 1) {
+      const int p = q >> 1;   // below 64
+      const uint32_t pk = rlane(t0, p);
+      if (!(pk > t)) break;
+      put(q, pk, rlane(n0, p));
+      q = p;
+    }
+    put(q, t, n);
+  }
   BPSX_DEV void push(uint32_t t, uint32_t n, int lane) {
     size++;
+#ifndef BPSX_SCALAR_SIFT
     bubble_up(size, t, n, lane);
+#else
+    sift_up(size, t, n);
+#endif
   }
   // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
+    const int q = position(n, lane);
+    if (!q) return;
+#ifndef BPSX_SCALAR_SIFT
+    bubble_up(q, t, n, lane);
+#else
+    sift_up(q, t, n);
+#endif
+  }
+  // heap position of node n's entry, 0 if it has none
+  BPSX_DEV int position(uint32_t n, int lane) const {
     const unsigned long long m0 = __ballot(lane >= 1 && lane <= size && n0 == n);
-    const unsigned long long m1 = m0 ? 0ull : __ballot(64 + lane <= size && n1 == n);
-    if (!(m0 | m1)) return;
-    const int q = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
+    if (m0) return __ffsll((long long)m0) - 1;
+    if (size < 64) return 0;
+    const unsigned long long m1 = __ballot(64 + lane <= size && n1 == n);
+    return m1 ? 64 + __ffsll((long long)m1) - 1 : 0;
+  }
+  // push (open false) or modify (open true) through one copy of the walk; an open node without
+  // an entry (there is none) would be a walk from position 0, which changes nothing
+  BPSX_DEV void update(bool open, uint32_t n, uint32_t t, int lane) {
+    int q;
+    if (open) q = position(n, lane);
+    else q = ++size;
     bubble_up(q, t, n, lane);
   }
   // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
   // by the root down to a leaf along the smaller children and then bubbles the former last
-  // entry up from there; along that route keys never decrease, so the entry ends up above
-  // the first route element greater than it and nothing below moves.  Which child the hole
-  // moves to depends only on the children's keys, which the moves above them do not change:
-  // every lane q picks the smaller child of position q (cross-lane reads; positions past the
-  // end hold kEmpty), the route is read off that table with dependent lane reads, and then
-  // every route position whose smaller child is not greater than the entry takes that child,
-  // and the first one whose child is greater takes the entry.
+  // entry up from there; along that route keys never decrease, so the entry ends up above the
+  // first route element greater than it and nothing below moves.  Which child the hole moves to
+  // depends only on the children's keys, which the moves above them do not change, so the
+  // route is known at once: siblings sit in neighbouring lanes, one comparison with the
+  // neighbour says for every position whether it is the smaller of its pair (the left one when
+  // equal), and a position is on the route when that holds for itself and all its ancestors,
+  // a test of the ballot against a per-lane constant.  Then every route position whose
+  // smaller child is not greater than the entry takes that child, and the first one whose
+  // child is greater takes the entry.  Positions past the end hold kEmpty and never move.
   BPSX_DEV void pop(int lane) {
     const int last = size;
     size--;
@@ -179,40 +237,35 @@ struct RegHeap {
     if (size == 0) return;
     const bool wide = size >= 64;           // entries in the second pair
     const bool lo = lane < 32;              // children of positions 32..63 are in the second pair
+    constexpr unsigned long long kOdd = 0xaaaaaaaaaaaaaaaaull;
+    // less0: the position's key is below its sibling's.  A right child is the smaller one when
+    // that holds, a left child unless it holds for its right neighbour.
+    const unsigned long long less0 = __ballot(t0 < quad_swap(t0));
+    const unsigned long long lose0 = ~((less0 & kOdd) | (~(less0 >> 1) & ~kOdd));
+    unsigned long long less1 = 0;
+    if (wide) less1 = __ballot(t1 < quad_swap(t1));
+    const bool on = lane >= 1 && ((anc0 & (uint32_t)lose0) | (anc1 & (uint32_t)(lose0 >> 32))) == 0;
+    // the smaller child of this lane's position: the right one if its key is below the left one's
     const int c0 = (2 * lane) & 63;
-    // keys and nodes of both children in one round of cross-lane reads
-    uint32_t cl = xlane(c0, t0), cr = xlane(c0 + 1, t0);
-    uint32_t nl = xlane(c0, n0), nr = xlane(c0 + 1, n0);
+    const unsigned long long lessc = lo ? less0 : less1;
+    const int c = c0 + (int)((uint32_t)(lessc >> (c0 + 1)) & 1u);
+    uint32_t ck = xlane(c, t0), cn = xlane(c, n0);
     if (wide) {
-      const uint32_t hl = xlane(c0, t1), hr = xlane(c0 + 1, t1), ml = xlane(c0, n1), mr = xlane(c0 + 1, n1);
-      cl = lo ? cl : hl; cr = lo ? cr : hr; nl = lo ? nl : ml; nr = lo ? nr : mr;
+      const uint32_t hk = xlane(c, t1), hn = xlane(c, n1);
+      ck = lo ? ck : hk; cn = lo ? cn : hn;
     } else {
-      cl = lo ? cl : kEmpty; cr = lo ? cr : kEmpty;
+      ck = lo ? ck : kEmpty;
     }
-    const bool right = cr < cl;
-    const uint32_t cmin = right ? cr : cl;
-    const uint32_t cn = right ? nr : nl;
-    const uint32_t choice = (uint32_t)(2 * lane) + (right ? 1u : 0u);   // position 2..127
-    // route of the hole: 1, choice[1], choice[choice[1]], ...
-    unsigned long long route = 2ull;
-    uint32_t q = 1;
-#pragma unroll
-    for (int lvl = 0; lvl < 5; ++lvl) {
-      q = rlane(choice, (int)(q & 31));     // levels 0..4 start from positions below 32
-      route |= 1ull << (q & 63);
-    }
-    const bool on = (route >> lane) & 1ull;
-    const bool take = on && cmin <= lt;
+    const bool take = on && ck <= lt;
     const bool land = on && !take && (lane == 1 || t0 <= lt);
     if (wide) {
-      // sixth level: from position q in 32..63 to its smaller child in the second pair, which has
-      // no children of its own: it takes the entry if its parent took it
-      const uint32_t e = rlane(choice, (int)(q & 63));
-      const bool here = lane == (int)(e & 63) && t1 <= lt;
+      // positions 64..127 have no children: the one on the route takes the entry if its parent took it
+      const unsigned long long lose1 = ~((less1 & kOdd) | (~(less1 >> 1) & ~kOdd));
+      const bool here = ((lose1 >> lane) & 1ull) == 0 && ((panc0 & (uint32_t)lose0) | (panc1 & (uint32_t)(lose0 >> 32))) == 0 && t1 <= lt;
       t1 = here ? lt : t1;
       n1 = here ? ln : n1;
     }
-    t0 = take ? cmin : (land ? lt : t0);
+    t0 = take ? ck : (land ? lt : t0);
     n0 = take ? cn : (land ? ln : n0);
   }
 };
@@ -615,6 +668,212 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
   return kAstarEmpty;
 }
 
+// The same loop for an open list in registers (S as above), two nodes per pass.  Besides the
+// node at the root (A, lanes 0..5) the pass works on the smaller child of the root (B, lanes
+// 16..21), which is what the reference pops next unless A's expansion puts something smaller
+// on the list: the edge records of both arrive in one load, and node lookup, costs, node
+// creation and stores of both are done by the same instructions.  B's results are computed
+// from the state before A's expansion; they are what the reference computes after it when
+//   - every total A puts on the open list is at least B's (B stays at the root: an entry
+//     moves past its parent only when its key is smaller),
+//   - A created or updated no node that B read (a neighbour of both) and not B's own node
+//     (A's own node is closed before either looks anything up, as it is when B's turn comes),
+// and B is not the goal.  Then the pass applies A's and B's updates in the reference's order:
+// new nodes take consecutive indices, A's first; the "nearest so far" record and the open
+// list see A's updates in edge order, then B's pop, then B's updates.  Otherwise B's lanes
+// are dropped and B becomes A of the next pass.
+template <bool S>
+BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
+#ifdef BPSX_PHASE_TIMING
+                               , unsigned long long* phase_acc, unsigned long long& phase_t0
+#endif
+                               ) {
+  const int lane = g.lane;
+  GeoLds* L = g.L;
+  const float H_SCALE = 0.999f;
+  const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
+  endIp = (uint32_t)uniform_i((int)endIp);
+  RegHeap& rh = st.rh;
+  const bool rowB = lane >= 16;
+  const int el = lane & 15;                      // edge handled by this lane
+  const bool edgeLane = el < kNvp && lane < 32;
+  while (rh.size > 0) {
+    if (!S && g.nodeCount > kLinksLds - 2 * kNvp) return kAstarGrowLinks;
+    if (rh.size > kRegHeap - 2 * kNvp) return kAstarGrowHeap;
+    const uint32_t rootA = rlane(rh.n0, 1);
+    const int biA = (int)(rootA & 0x7ffu);
+    const uint32_t ipA = rootA >> 11;
+    const uint32_t kl = rlane(rh.t0, 2), kr = rlane(rh.t0, 3);   // kEmpty past the end
+    const uint32_t rootB = kr < kl ? rlane(rh.n0, 3) : rlane(rh.n0, 2);
+    const uint32_t keyB = kr < kl ? kr : kl;
+    const int biB = (int)(rootB & 0x7ffu);
+    const uint32_t ipB = rootB >> 11;
+    const bool spec = rh.size >= 2 && ipA != endIp && ipB != endIp;
+    const uint32_t blinkA = g.link<S>(biA);
+    const uint32_t blinkB = g.link<S>(spec ? biB : biA);   // unchanged by A whenever B is committed
+    const bool act = edgeLane && (!rowB || spec);
+    const int bi = (rowB && spec) ? biB : biA;   // the node this lane expands
+    uint32_t nb = kNoNb;
+    float m0 = 0, m1 = 0, m2 = 0;
+    if (act) {
+      const AEdge e = edges[(rowB ? ipB : ipA) * kNvp + (uint32_t)el];
+      nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
+    }
+    float b0, b1, b2, bcost;
+    uint32_t bparent;
+    {
+      const int w = bi & (kWindow - 1);
+      const bool binw = g.in_window(bi);
+      b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
+      bparent = L->w_parent[w];
+      if (__ballot(!binw)) {
+        if (!binw) {
+          BPSX_KEEP_APART();
+          const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
+          b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
+          bparent = g.ws->nodes[bi].parent;
+          BPSX_KEEP_APART();
+        }
+      }
+    }
+    PHASE_MARK(0);
+    rh.pop(lane);
+    PHASE_MARK(1);
+    g.set_link<S>(biA, with_flags(blinkA, 2u));   // open -> closed
+    if (ipA == endIp) { st.lastBest = biA; return kAstarGoal; }
+    (*pops)++;
+    PHASE_MARK(2);
+    const uint32_t bucket = GeoWave::hash(nb);
+    uint32_t chainHead, hitLink;
+    int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
+    // the polygon the expanded node was reached from is not entered again
+    if (bparent && ni + 1 == (int)bparent) nb = kNoNb;
+    PHASE_MARK(3);
+    // ---- costs of both nodes' steps (new nodes have no index yet and read slot 0)
+    const bool isNew = nb != kNoNb && ni < 0;
+    const bool valid = nb != kNoNb;
+    const int nis = (valid && !isNew) ? ni : 0;
+    const int rw = nis & (kWindow - 1);
+    uint32_t fl = link_flags(hitLink);
+    float p0 = L->w_pos[0][rw], p1 = L->w_pos[1][rw], p2 = L->w_pos[2][rw], oldTotal = L->w_total[rw];
+    const bool miss = valid && !isNew && !g.in_window(nis);
+    if (__ballot(miss)) {
+      if (miss) {
+        const ANode& hn = g.ws->nodes[nis];
+        BPSX_KEEP_APART();
+        const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
+        p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = hn.total;
+        BPSX_KEEP_APART();
+      }
+    }
+    if (isNew) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }
+    const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
+    const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
+    const float cc = cx * cx + cy * cy + cz * cz, ee = ex * ex + ey * ey + ez * ez;
+    const float roots = sqrt_exact(lanes_up8(cc, ee));
+    const float curCost = roots * 1.0f;
+    const float toEnd = lanes_down8(roots);
+    const bool last = nb == endIp;
+    const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
+    const float heuristic = last ? 0.0f : toEnd * H_SCALE;
+    const float total = cost + heuristic;
+    bool update = valid && !(fl && total >= oldTotal);
+    // ---- does B stand?
+    bool two = false;
+    if (spec) {
+      const uint32_t anb = (update && !rowB) ? nb : kNoNb;   // a lane of A that updates nothing leaves its node as B saw it
+      const uint32_t bnb = (valid && rowB) ? nb : kNoNb - 1u;   // never equal to anb of an idle lane
+      uint32_t clash = (uint32_t)(!rowB && update) & ((uint32_t)(__float_as_uint(total) < keyB) | (uint32_t)(nb == ipB));
+#pragma unroll
+      for (int j = 0; j < kNvp; ++j) clash |= (uint32_t)(bnb == rlane(anb, j));
+      two = !__ballot(clash != 0);
+    }
+    if (!two) update = update && !rowB;
+    const bool wasOpen = update && (fl & 1u) != 0;
+    PHASE_MARK(4);
+    // ---- new nodes take consecutive indices in edge order, A's before B's
+    {
+      const bool mine = isNew && update;   // a new node is always taken
+      const unsigned long long need = __ballot(mine);
+      if (need) {
+        const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
+        const int count = __popcll(need);
+        const int want = g.nodeCount + count;
+        // the reference carries on without the nodes that do not fit, but reports anything found
+        // after that as failure (only plain DT_SUCCESS counts, PathFinder.cpp:506): stop
+        if (S && want > kMaxNodes) { st.outOfNodes = true; return kAstarEmpty; }
+        if (mine) ni = g.nodeCount + rank;
+        g.nodeCount = want;
+        // All insert at once in front of the chain head their lookup saw.  Of several that share a
+        // bucket one store wins; the others see that when they read the head back and go round
+        // again behind the winner.  One new node needs no check.
+        bool pending = mine;
+        uint32_t head = chainHead;
+        for (;;) {
+          if (pending) {
+            g.set_link<S>(ni, make_link(nb, 1u, head));
+            L->first[bucket] = (uint16_t)ni;
+          }
+          wave_sync();
+          if (count == 1) break;
+          if (pending) {
+            head = L->first[bucket];
+            pending = head != (uint32_t)ni;
+          }
+          wave_sync();
+          if (!__ballot(pending)) break;
+        }
+      }
+    }
+    if (update) {
+      ANode& hn = g.ws->nodes[ni];
+      const int w = ni & (kWindow - 1);
+      const uint32_t parent = (uint32_t)bi + 1u;
+      if (!isNew) g.set_link<S>(ni, with_flags(hitLink, 1u));   // open (again)
+      if (g.in_window(ni)) {
+        L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2;
+        L->w_cost[w] = cost; L->w_total[w] = total;
+        L->w_parent[w] = (uint16_t)parent;
+      }
+      *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
+      *reinterpret_cast<uint2*>(&hn.total) = make_uint2(__float_as_uint(total), parent);
+    }
+    wave_sync();
+    PHASE_MARK(5);
+    // ---- ordered phase, in the reference's order: A's lanes come before B's.  First the
+    // "nearest so far" record (lastBestNode of findPath), then the open list.
+    const uint32_t packed = (uint32_t)ni | (nb << 11);
+    unsigned long long better = __ballot(update && heuristic < st.lastBestCost);
+    while (better) {
+      const int src = __ffsll((long long)better) - 1;
+      better &= better - 1;
+      const float h = lane_f(heuristic, src);
+      if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
+    }
+    const unsigned long long upd = __ballot(update);
+    const unsigned long long openMask = __ballot(wasOpen);
+    auto apply = [&](unsigned long long m) {
+      while (m) {
+        const int src = __ffsll((long long)m) - 1;
+        m &= m - 1;
+        rh.update((openMask >> src) & 1ull, rlane(packed, src), __float_as_uint(lane_f(total, src)), lane);
+      }
+    };
+    apply(upd & 0xffffull);
+    if (two) {   // A's updates are in: B leaves the open list
+      rh.pop(lane);
+      g.set_link<S>(biB, with_flags(blinkB, 2u));
+      (*pops)++;
+#ifdef BPSX_PHASE_TIMING
+      phase_acc[7]++;   // passes that expanded two nodes
+#endif
+      apply(upd & ~0xffffull);
+    }
+    PHASE_MARK(6);
+  }
+  return kAstarEmpty;
+}
+
 // Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
 // when the reference would report anything but plain DT_SUCCESS.
 BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev& s, uint32_t startIp, uint32_t endIp,
@@ -635,9 +894,14 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
   AstarState st;
   const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kNvp;
 #ifdef BPSX_PHASE_TIMING
-#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops, phase_acc, phase_t0)
+#define ASTAR_ARGS g, st, edges, endIp, endPos, pops, phase_acc, phase_t0
 #else
-#define ASTAR_RUN(M) astar_loop<M>(g, st, edges, endIp, endPos, pops)
+#define ASTAR_ARGS g, st, edges, endIp, endPos, pops
+#endif
+#ifdef BPSX_ONE_NODE_PER_PASS
+#define ASTAR_RUN(M) astar_loop<M>(ASTAR_ARGS)
+#else
+#define ASTAR_RUN(M) ((M) == 2 ? astar_loop<2>(ASTAR_ARGS) : astar_loop2<(M) == 1>(ASTAR_ARGS))
 #endif
   g.clear();
   {
@@ -659,7 +923,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.lastBest = 0;
     st.lastBestCost = total;
     st.outOfNodes = false;
-    st.rh.init();
+    st.rh.init(lane);
     st.rh.push(__float_as_uint(total), startIp << 11, lane);
   }
   AstarExit ex = ASTAR_RUN(0);
@@ -680,6 +944,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     ex = ASTAR_RUN(2);
   }
 #undef ASTAR_RUN
+#undef ASTAR_ARGS
   (void)ex;
   if (st.outOfNodes) return 0;   // no path to build: the result is a failure
   const int lastBest = st.lastBest;
