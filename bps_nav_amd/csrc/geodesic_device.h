@@ -62,6 +62,8 @@ BPSX_DEV void set_wave_priority(int p) {
   else if (p == 1) __builtin_amdgcn_s_setprio(1);
   else __builtin_amdgcn_s_setprio(0);
 }
+// mask of the lanes where b holds (takes the condition as such, not widened to an integer and compared again)
+BPSX_DEV unsigned long long lanes_where(bool b) { return __builtin_amdgcn_ballot_w64(b); }
 BPSX_DEV int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
 BPSX_DEV float uniform_f(float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); }
 BPSX_DEV float lane_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
@@ -91,7 +93,7 @@ BPSX_DEV float lanes_down8(float v) {
 // between takes the library routine.
 BPSX_DEV float sqrt_exact(float x) {
   const uint32_t xb = __float_as_uint(x);
-  if (__builtin_expect(__ballot(xb - 1u < 0x0f800000u - 1u) != 0, 0)) return sqrtf(x);   // 0 < x < 2^-96 in some lane: never in practice
+  if (__builtin_expect(lanes_where(xb - 1u < 0x0f800000u - 1u) != 0, 0)) return sqrtf(x);   // 0 < x < 2^-96 in some lane: never in practice
   const float s = __builtin_amdgcn_sqrtf(x);
   const float down = __uint_as_float(__float_as_uint(s) - 1u), up = __uint_as_float(__float_as_uint(s) + 1u);
   const float rdown = fmaf(-down, s, x), rup = fmaf(-up, s, x);
@@ -167,46 +169,21 @@ struct RegHeap {
     t0 = parentMoves ? pk : (land ? t : t0);
     n0 = parentMoves ? pn : (land ? n : n0);
   }
-  // The same walk on the scalar unit: q, t and n are wave-uniform, the parents' keys are read
-  // with lane reads, and an entry of A* mostly stays where it is put or moves a level or two.
-  BPSX_DEV void put(int q, uint32_t t, uint32_t n) {
-    if (q < 64) { t0 = wlane(t0, t, q); n0 = wlane(n0, n, q); }
-    else { t1 = wlane(t1, t, q & 63); n1 = wlane(n1, n, q & 63); }
-  }
-  BPSX_DEV void sift_up(int q, uint32_t t, uint32_t n) {
-    while (q > 1) {
-      const int p = q >> 1;   // below 64
-      const uint32_t pk = rlane(t0, p);
-      if (!(pk > t)) break;
-      put(q, pk, rlane(n0, p));
-      q = p;
-    }
-    put(q, t, n);
-  }
   BPSX_DEV void push(uint32_t t, uint32_t n, int lane) {
     size++;
-#ifndef BPSX_SCALAR_SIFT
     bubble_up(size, t, n, lane);
-#else
-    sift_up(size, t, n);
-#endif
   }
   // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
   BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
     const int q = position(n, lane);
-    if (!q) return;
-#ifndef BPSX_SCALAR_SIFT
-    bubble_up(q, t, n, lane);
-#else
-    sift_up(q, t, n);
-#endif
+    if (q) bubble_up(q, t, n, lane);
   }
   // heap position of node n's entry, 0 if it has none
   BPSX_DEV int position(uint32_t n, int lane) const {
-    const unsigned long long m0 = __ballot(lane >= 1 && lane <= size && n0 == n);
+    const unsigned long long m0 = lanes_where(lane >= 1 && lane <= size && n0 == n);
     if (m0) return __ffsll((long long)m0) - 1;
     if (size < 64) return 0;
-    const unsigned long long m1 = __ballot(64 + lane <= size && n1 == n);
+    const unsigned long long m1 = lanes_where(64 + lane <= size && n1 == n);
     return m1 ? 64 + __ffsll((long long)m1) - 1 : 0;
   }
   // push (open false) or modify (open true) through one copy of the walk; an open node without
@@ -240,10 +217,10 @@ struct RegHeap {
     constexpr unsigned long long kOdd = 0xaaaaaaaaaaaaaaaaull;
     // less0: the position's key is below its sibling's.  A right child is the smaller one when
     // that holds, a left child unless it holds for its right neighbour.
-    const unsigned long long less0 = __ballot(t0 < quad_swap(t0));
+    const unsigned long long less0 = lanes_where(t0 < quad_swap(t0));
     const unsigned long long lose0 = ~((less0 & kOdd) | (~(less0 >> 1) & ~kOdd));
     unsigned long long less1 = 0;
-    if (wide) less1 = __ballot(t1 < quad_swap(t1));
+    if (wide) less1 = lanes_where(t1 < quad_swap(t1));
     const bool on = lane >= 1 && ((anc0 & (uint32_t)lose0) | (anc1 & (uint32_t)(lose0 >> 32))) == 0;
     // the smaller child of this lane's position: the right one if its key is below the left one's
     const int c0 = (2 * lane) & 63;
@@ -386,7 +363,7 @@ struct GeoWave {
     *head = cur;
     int found = -1;
     uint32_t fl = 0;
-    while (__ballot(cur != kChainEnd)) {
+    while (lanes_where(cur != kChainEnd)) {
       const bool live = cur != kChainEnd;
       const uint32_t l = link<S>(live ? (int)cur : 0);
       const bool hit = live && link_id(l) == ip;
@@ -436,7 +413,7 @@ struct GeoWave {
     int found = -1;
     for (int base = 0; base < heapSize; base += 64) {
       const int i = base + lane;
-      const unsigned long long m = __ballot(i < heapSize && (int)hget<S>(i).node == n);
+      const unsigned long long m = lanes_where(i < heapSize && (int)hget<S>(i).node == n);
       if (m) { found = base + (__ffsll((long long)m) - 1); break; }
     }
     if (found >= 0) bubble_up<S>(found, t, n);
@@ -549,7 +526,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     PHASE_MARK(3);
     // new nodes take consecutive indices in edge order; past the pool's end they are dropped
     const bool isNew = nb != kNoNb && ni < 0;
-    const unsigned long long need = __ballot(isNew);
+    const unsigned long long need = lanes_where(isNew);
     if (need) {
       const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
       const int count = __popcll(need);
@@ -581,12 +558,12 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
           pending = head != (uint32_t)ni;
         }
         wave_sync();
-        if (!__ballot(pending)) break;
+        if (!lanes_where(pending)) break;
       }
     }
     PHASE_MARK(4);
 #ifdef BPSX_QUERY_TRACE
-    g.missNb += (uint32_t)__popcll(__ballot(nb != kNoNb && !isNew && !g.in_window(ni)));
+    g.missNb += (uint32_t)__popcll(lanes_where(nb != kNoNb && !isNew && !g.in_window(ni)));
 #endif
     // Costs of the step to each neighbour (lane-wise).  Written with few branches: all lanes
     // issue the one round of LDS reads a revisited node needs (idle lanes read slot 0; its flags
@@ -601,7 +578,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     uint32_t fl = link_flags(hitLink);
     float p0 = L->w_pos[0][w], p1 = L->w_pos[1][w], p2 = L->w_pos[2][w], oldTotal = L->w_total[w];
     const bool miss = valid && !isNew && !inw;
-    if (__ballot(miss)) {
+    if (lanes_where(miss)) {
       if (miss) {
         BPSX_KEEP_APART();
         const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
@@ -639,7 +616,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     // findPath): an update replaces it when its heuristic is lower; only lanes below the
     // current record can matter, usually none.
     const uint32_t packed = (uint32_t)ni | (nb << 11);   // heap entry of this lane's node
-    unsigned long long better = __ballot(update && heuristic < st.lastBestCost);
+    unsigned long long better = lanes_where(update && heuristic < st.lastBestCost);
     while (better) {
       const int src = __ffsll((long long)better) - 1;
       better &= better - 1;
@@ -647,8 +624,8 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
     }
     // then the open list
-    unsigned long long upd = __ballot(update);
-    const unsigned long long openMask = __ballot(wasOpen);
+    unsigned long long upd = lanes_where(update);
+    const unsigned long long openMask = lanes_where(wasOpen);
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
@@ -726,7 +703,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       const bool binw = g.in_window(bi);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
       bparent = L->w_parent[w];
-      if (__ballot(!binw)) {
+      if (lanes_where(!binw)) {
         if (!binw) {
           BPSX_KEEP_APART();
           const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
@@ -757,7 +734,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     uint32_t fl = link_flags(hitLink);
     float p0 = L->w_pos[0][rw], p1 = L->w_pos[1][rw], p2 = L->w_pos[2][rw], oldTotal = L->w_total[rw];
     const bool miss = valid && !isNew && !g.in_window(nis);
-    if (__ballot(miss)) {
+    if (lanes_where(miss)) {
       if (miss) {
         const ANode& hn = g.ws->nodes[nis];
         BPSX_KEEP_APART();
@@ -786,7 +763,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       uint32_t clash = (uint32_t)(!rowB && update) & ((uint32_t)(__float_as_uint(total) < keyB) | (uint32_t)(nb == ipB));
 #pragma unroll
       for (int j = 0; j < kNvp; ++j) clash |= (uint32_t)(bnb == rlane(anb, j));
-      two = !__ballot(clash != 0);
+      two = !lanes_where(clash != 0);
     }
     if (!two) update = update && !rowB;
     const bool wasOpen = update && (fl & 1u) != 0;
@@ -794,7 +771,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     // ---- new nodes take consecutive indices in edge order, A's before B's
     {
       const bool mine = isNew && update;   // a new node is always taken
-      const unsigned long long need = __ballot(mine);
+      const unsigned long long need = lanes_where(mine);
       if (need) {
         const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
         const int count = __popcll(need);
@@ -821,7 +798,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
             pending = head != (uint32_t)ni;
           }
           wave_sync();
-          if (!__ballot(pending)) break;
+          if (!lanes_where(pending)) break;
         }
       }
     }
@@ -843,15 +820,15 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     // ---- ordered phase, in the reference's order: A's lanes come before B's.  First the
     // "nearest so far" record (lastBestNode of findPath), then the open list.
     const uint32_t packed = (uint32_t)ni | (nb << 11);
-    unsigned long long better = __ballot(update && heuristic < st.lastBestCost);
+    unsigned long long better = lanes_where(update && heuristic < st.lastBestCost);
     while (better) {
       const int src = __ffsll((long long)better) - 1;
       better &= better - 1;
       const float h = lane_f(heuristic, src);
       if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
     }
-    const unsigned long long upd = __ballot(update);
-    const unsigned long long openMask = __ballot(wasOpen);
+    const unsigned long long upd = lanes_where(update);
+    const unsigned long long openMask = lanes_where(wasOpen);
     auto apply = [&](unsigned long long m) {
       while (m) {
         const int src = __ffsll((long long)m) - 1;
@@ -987,7 +964,7 @@ BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const S
     p[0] = l[0]; p[1] = l[1]; p[2] = l[2]; p[3] = rr[0]; p[4] = rr[1]; p[5] = rr[2];
   }
   wave_sync();
-  if (__ballot(missing)) return INF;
+  if (lanes_where(missing)) return INF;
   float cs[3], ce[3];
   closest_on_poly_boundary(nav.polys[s.poly_base + F->corridor[0]], startPos, cs);
   closest_on_poly_boundary(nav.polys[s.poly_base + F->corridor[n - 1]], endPos, ce);
