@@ -153,14 +153,14 @@ struct RegHeap {
   // one step down that way (they form a run from q upwards: keys never increase towards the
   // root) and the entry lands on top of the run.  Positions 64..127 have all their ancestors
   // in the first pair, so only q itself can be in the second.
-  BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n, int lane) {
+  template <bool W = true> BPSX_DEV void bubble_up(int q, uint32_t t, uint32_t n, int lane) {
     const int up = (31 - __clz(q)) - (31 - __clz(lane));   // lane 0 (clz 32) is no heap position
     const bool on = lane >= 1 && up >= 0 && (q >> (up & 31)) == lane;
     const uint32_t pk = xlane(lane >> 1, t0), pn = xlane(lane >> 1, n0);
     const bool parentMoves = on && lane > 1 && pk > t;
     const bool vacant = lane == q || t0 > t;
     const bool land = on && vacant && !parentMoves;
-    if (q >= 64) {
+    if (W && q >= 64) {
       const uint32_t qk = rlane(t0, q >> 1), qn = rlane(n0, q >> 1);
       const bool here = lane == (q & 63);
       t1 = here ? (qk > t ? qk : t) : t1;
@@ -179,20 +179,20 @@ struct RegHeap {
     if (q) bubble_up(q, t, n, lane);
   }
   // heap position of node n's entry, 0 if it has none
-  BPSX_DEV int position(uint32_t n, int lane) const {
+  template <bool W = true> BPSX_DEV int position(uint32_t n, int lane) const {
     const unsigned long long m0 = lanes_where(lane >= 1 && lane <= size && n0 == n);
     if (m0) return __ffsll((long long)m0) - 1;
-    if (size < 64) return 0;
+    if (!W || size < 64) return 0;
     const unsigned long long m1 = lanes_where(64 + lane <= size && n1 == n);
     return m1 ? 64 + __ffsll((long long)m1) - 1 : 0;
   }
   // push (open false) or modify (open true) through one copy of the walk; an open node without
   // an entry (there is none) would be a walk from position 0, which changes nothing
-  BPSX_DEV void update(bool open, uint32_t n, uint32_t t, int lane) {
+  template <bool W = true> BPSX_DEV void update(bool open, uint32_t n, uint32_t t, int lane) {
     int q;
-    if (open) q = position(n, lane);
+    if (open) q = position<W>(n, lane);
     else q = ++size;
-    bubble_up(q, t, n, lane);
+    bubble_up<W>(q, t, n, lane);
   }
   // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
   // by the root down to a leaf along the smaller children and then bubbles the former last
@@ -205,14 +205,15 @@ struct RegHeap {
   // a test of the ballot against a per-lane constant.  Then every route position whose
   // smaller child is not greater than the entry takes that child, and the first one whose
   // child is greater takes the entry.  Positions past the end hold kEmpty and never move.
-  BPSX_DEV void pop(int lane) {
+  // W false: the caller knows that the list has fewer than 64 entries.
+  template <bool W = true> BPSX_DEV void pop(int lane) {
     const int last = size;
     size--;
     uint32_t lt, ln;
-    if (last < 64) { lt = rlane(t0, last); ln = rlane(n0, last); t0 = wlane(t0, kEmpty, last); }
+    if (!W || last < 64) { lt = rlane(t0, last); ln = rlane(n0, last); t0 = wlane(t0, kEmpty, last); }
     else { lt = rlane(t1, last & 63); ln = rlane(n1, last & 63); t1 = wlane(t1, kEmpty, last & 63); }
     if (size == 0) return;
-    const bool wide = size >= 64;           // entries in the second pair
+    const bool wide = W && size >= 64;      // entries in the second pair
     const bool lo = lane < 32;              // children of positions 32..63 are in the second pair
     constexpr unsigned long long kOdd = 0xaaaaaaaaaaaaaaaaull;
     // less0: the position's key is below its sibling's.  A right child is the smaller one when
@@ -659,7 +660,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
 // new nodes take consecutive indices, A's first; the "nearest so far" record and the open
 // list see A's updates in edge order, then B's pop, then B's updates.  Otherwise B's lanes
 // are dropped and B becomes A of the next pass.
-template <bool S>
+template <bool S, bool W>
 BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
 #ifdef BPSX_PHASE_TIMING
                                , unsigned long long* phase_acc, unsigned long long& phase_t0
@@ -676,7 +677,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
   const bool edgeLane = el < kNvp && lane < 32;
   while (rh.size > 0) {
     if (!S && g.nodeCount > kLinksLds - 2 * kNvp) return kAstarGrowLinks;
-    if (rh.size > kRegHeap - 2 * kNvp) return kAstarGrowHeap;
+    if (rh.size > (W ? kRegHeap : 63) - 2 * kNvp) return kAstarGrowHeap;   // W false: all entries in the first register pair
     const uint32_t rootA = rlane(rh.n0, 1);
     const int biA = (int)(rootA & 0x7ffu);
     const uint32_t ipA = rootA >> 11;
@@ -714,7 +715,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       }
     }
     PHASE_MARK(0);
-    rh.pop(lane);
+    rh.template pop<W>(lane);
     PHASE_MARK(1);
     g.set_link<S>(biA, with_flags(blinkA, 2u));   // open -> closed
     if (ipA == endIp) { st.lastBest = biA; return kAstarGoal; }
@@ -833,12 +834,12 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       while (m) {
         const int src = __ffsll((long long)m) - 1;
         m &= m - 1;
-        rh.update((openMask >> src) & 1ull, rlane(packed, src), __float_as_uint(lane_f(total, src)), lane);
+        rh.template update<W>((openMask >> src) & 1ull, rlane(packed, src), __float_as_uint(lane_f(total, src)), lane);
       }
     };
     apply(upd & 0xffffull);
     if (two) {   // A's updates are in: B leaves the open list
-      rh.pop(lane);
+      rh.template pop<W>(lane);
       g.set_link<S>(biB, with_flags(blinkB, 2u));
       (*pops)++;
 #ifdef BPSX_PHASE_TIMING
@@ -875,11 +876,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #else
 #define ASTAR_ARGS g, st, edges, endIp, endPos, pops
 #endif
-#ifdef BPSX_ONE_NODE_PER_PASS
 #define ASTAR_RUN(M) astar_loop<M>(ASTAR_ARGS)
-#else
-#define ASTAR_RUN(M) ((M) == 2 ? astar_loop<2>(ASTAR_ARGS) : astar_loop2<(M) == 1>(ASTAR_ARGS))
-#endif
   g.clear();
   {
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
@@ -903,8 +900,22 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.rh.init(lane);
     st.rh.push(__float_as_uint(total), startIp << 11, lane);
   }
+#ifdef BPSX_ONE_NODE_PER_PASS
   AstarExit ex = ASTAR_RUN(0);
   if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
+#else
+  // the loop is instantiated for links in LDS only or spilling, and for an open list within one
+  // register pair or two; a search moves on when one more pass could outgrow what it runs in
+  AstarExit ex;
+  bool spill = false, wide = false;
+  for (;;) {
+    if (!spill) ex = wide ? astar_loop2<false, true>(ASTAR_ARGS) : astar_loop2<false, false>(ASTAR_ARGS);
+    else ex = wide ? astar_loop2<true, true>(ASTAR_ARGS) : astar_loop2<true, false>(ASTAR_ARGS);
+    if (ex == kAstarGrowLinks) { g.linkSpills++; spill = true; }
+    else if (ex == kAstarGrowHeap && !wide) wide = true;
+    else break;
+  }
+#endif
   if (ex == kAstarGrowHeap) {
     g.heapSpills++;
     // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
