@@ -682,7 +682,8 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     const int biA = (int)(rootA & 0x7ffu);
     const uint32_t ipA = rootA >> 11;
     const uint32_t kl = rlane(rh.t0, 2), kr = rlane(rh.t0, 3);   // kEmpty past the end
-    const uint32_t rootB = kr < kl ? rlane(rh.n0, 3) : rlane(rh.n0, 2);
+    const uint32_t nl = rlane(rh.n0, 2), nr = rlane(rh.n0, 3);
+    const uint32_t rootB = kr < kl ? nr : nl;
     const uint32_t keyB = kr < kl ? kr : kl;
     const int biB = (int)(rootB & 0x7ffu);
     const uint32_t ipB = rootB >> 11;
@@ -766,7 +767,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       for (int j = 0; j < kNvp; ++j) clash |= (uint32_t)(bnb == rlane(anb, j));
       two = !lanes_where(clash != 0);
     }
-    if (!two) update = update && !rowB;
+    update = update & (!rowB | two);   // B's lanes are dropped unless B stands
     const bool wasOpen = update && (fl & 1u) != 0;
     PHASE_MARK(4);
     // ---- new nodes take consecutive indices in edge order, A's before B's
