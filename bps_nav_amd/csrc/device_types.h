@@ -140,9 +140,24 @@ struct HeapEntry {
 
 // HBM slot of one A* wavefront: the node pool (LDS caches its hot part) and the open-list
 // entries beyond what LDS holds.
+// Record of the open-list operations of a search that keeps its open list sorted (see
+// geodesic_device.h): per pass one header (key = number of entries popped | number of records
+// that follow << 8, word = kOpHeader) followed by the pass's pushes and modifies in row and
+// edge order (key = total as bits, word = packed node | row of the pass << 26 | 1 << 28 if the
+// node was open).  A header with kOpUnordered says that the pass's first two rows had the same
+// total: the reference expanded them in the order its heap had them in, which the replay finds
+// out; the header's low 26 bits then name row 0's node.
+struct OpRec {
+  uint32_t key;
+  uint32_t word;
+};
+constexpr uint32_t kOpHeader = 0x80000000u, kOpUnordered = 0x40000000u;
+constexpr int kOpLogCap = 8192;
+
 struct alignas(128) GeoSlot {
   ANode nodes[kMaxNodes];
   HeapEntry heap_spill[kMaxNodes];
+  OpRec oplog[kOpLogCap];
 };
 
 struct GeoQuery {
@@ -176,7 +191,7 @@ constexpr uint32_t kCostUnknown = 0xffffffffu;
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,
-  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18   // 8..15: phase cycles of the diagnostic build
+  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18, kCntExactRuns = 19, kCntTieReplays = 20   // 8..15: phase cycles of the diagnostic build
 };
 
 }  // namespace bpsx

@@ -58,7 +58,7 @@ int dev_alloc(T** p, size_t count) {
 // GPU, held until the process ends: the queries built from the caller's arrays, the queue
 // counters, and the node pools of the kStaticBlocks * 2 wavefronts that serve the queue.
 namespace {
-constexpr uint32_t kStaticBlocks = 32;
+constexpr uint32_t kStaticBlocks = 16;
 constexpr size_t kStaticQueriesBytes = (size_t)BPSX_STATIC_MAX_QUERIES * sizeof(GeoQuery);
 constexpr size_t kStaticCountsBytes = 256;
 static_assert((kGeoClasses + 2) * sizeof(uint32_t) <= kStaticCountsBytes, "queue counters must fit their part");

@@ -188,10 +188,20 @@ struct RegHeap {
   }
   // push (open false) or modify (open true) through one copy of the walk; an open node without
   // an entry (there is none) would be a walk from position 0, which changes nothing
+  // Most entries stay where they start (a new total is rarely below its parent's): that case is
+  // two lane writes on the scalar unit's word, without the lane-parallel walk.
   template <bool W = true> BPSX_DEV void update(bool open, uint32_t n, uint32_t t, int lane) {
     int q;
     if (open) q = position<W>(n, lane);
     else q = ++size;
+#ifndef BPSX_NO_PUSH_FAST_PATH
+    const uint32_t pk = rlane(t0, q >> 1);   // position 0 holds kEmpty: no entry (q = 0) and the root take the walk
+    if (pk <= t) {
+      if (!W || q < 64) { t0 = wlane(t0, t, q); n0 = wlane(n0, n, q); }
+      else { t1 = wlane(t1, t, q & 63); n1 = wlane(n1, n, q & 63); }
+      return;
+    }
+#endif
     bubble_up<W>(q, t, n, lane);
   }
   // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
@@ -248,13 +258,134 @@ struct RegHeap {
   }
 };
 
-struct AstarState {
-  int lastBest;
-  float lastBestCost;
-  bool outOfNodes;
-  RegHeap rh;
+// The open list as a sorted array in registers.  dtNodeQueue::pop returns the entry with the
+// smallest total; while that smallest total is held by one entry only, which entry that is
+// does not depend on how the reference's binary heap happens to be arranged.  So a search can
+// keep its open list in any form that yields the minimum, as long as it notices when two
+// entries share the smallest total (a tie, about one pop in ten thousand) and then asks the
+// exact heap.  Sorted by total, entry i in lane i & 63 of pair i >> 6: the next nodes to expand
+// are the first lanes, a pop is a shift of all lanes by one, and an insertion is one comparison
+// of all lanes with the new total and a shift of those above it.  Unused places hold kEmpty
+// keys and kNone nodes.  Entries with equal totals sit next to each other in no defined order.
+struct OpenList {
+  uint32_t t0, n0, t1, n1;   // totals as bit patterns (see RegHeap), nodes packed like RegHeap's
+  int size;
+  static constexpr uint32_t kEmpty = 0x7fffffffu;
+  static constexpr uint32_t kNone = 0xffffffffu;    // no packed node looks like this (26 bits)
+  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = kNone; size = 0; }
+  // lane L takes v of lane L - 1, lane 0 keeps `first`
+  static BPSX_DEV uint32_t up1(uint32_t first, uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+  }
+  // lane L takes v of lane L + 1, lane 63 keeps `last`
+  static BPSX_DEV uint32_t down1(uint32_t last, uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)last, (int)v, 0x130 /* wave_shl:1 */, 0xf, 0xf, false);
+  }
+  // v as a select operand under a lane mask held in scalar registers
+  static BPSX_DEV uint32_t pick(unsigned long long mask, uint32_t yes, uint32_t no) {
+    uint32_t r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(mask));
+    return r;
+  }
+  // The first c entries leave (W false: the list lives in the first pair only).
+  template <bool W> BPSX_DEV void drop_front(int c, int lane) {
+    size -= c;
+    if (!W) {
+      for (int i = 0; i < c; ++i) { t0 = down1(kEmpty, t0); n0 = down1(kNone, n0); }
+    } else {
+      const int src = ((lane + c) & 63) * 4;
+      const uint32_t a0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)t0), b0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)n0);
+      const uint32_t a1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)t1), b1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)n1);
+      const bool same = lane + c < 64;
+      t0 = same ? a0 : a1; n0 = same ? b0 : b1;
+      t1 = same ? a1 : kEmpty; n1 = same ? b1 : kNone;
+    }
+  }
+  // push (open false) or modify (open true: the node's entry, if it still has one, leaves
+  // first) of node n with total t.  The entry goes behind those with totals up to t.
+  template <bool W> BPSX_DEV void update(bool open, uint32_t n, uint32_t t, int lane) {
+    unsigned long long m0 = lanes_where(t0 > t), m1 = W ? lanes_where(t1 > t) : 0ull;
+    int r = -1;
+    if (open) {
+      const unsigned long long h0 = lanes_where(n0 == n);
+      if (h0) r = __ffsll((long long)h0) - 1;
+      else if (W) { const unsigned long long h1 = lanes_where(n1 == n); if (h1) r = 64 + __ffsll((long long)h1) - 1; }
+    }
+    if (r >= 0) {
+      // only the entries from the new place up to the old one move
+      if (r < 64) { m0 &= (2ull << r) - 1ull; m1 = 0; }
+      else m1 &= (2ull << (r - 64)) - 1ull;
+    } else {
+      size++;
+    }
+    const int p = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
+    if (W) {
+      const uint32_t ct = rlane(t0, 63), cn = rlane(n0, 63);   // what moves up into the second pair
+      const uint32_t s1 = up1(ct, t1), u1 = up1(cn, n1);
+      t1 = pick(m1, s1, t1); n1 = pick(m1, u1, n1);
+    }
+    const uint32_t s0 = up1(t0, t0), u0 = up1(n0, n0);
+    t0 = pick(m0, s0, t0); n0 = pick(m0, u0, n0);
+    if (!W || p < 64) { t0 = wlane(t0, t, p); n0 = wlane(n0, n, p); }
+    else { t1 = wlane(t1, t, p - 64); n1 = wlane(n1, n, p - 64); }
+  }
 };
-enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3 };
+
+struct AstarState {
+  int lastBest;      // the goal's node once it has been popped
+  bool outOfNodes;
+  RegHeap rh;        // the reference's heap: always (exact loops), or as of log record `synced` (sorted-list loop)
+  OpenList ol;
+  int logEnd;        // records in the slot's operation log
+  int synced;        // records already applied to rh
+};
+
+// Applies log records [st.synced, st.logEnd) to the reference's heap, pass by pass.  Records are
+// fetched 64 at a time, one per lane; a pass has at most 1 + 4 * 6 records.  False when the heap
+// outgrows the registers.
+BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
+  RegHeap& rh = st.rh;
+  int base = st.synced;        // record held by lane 0
+  uint32_t rk = 0, rw = 0;
+  bool loaded = false;
+  for (int pos = st.synced; pos < st.logEnd;) {
+    if (!loaded || pos + 1 + 4 * kNvp > base + 64) {
+      base = pos;
+      rk = 0; rw = 0;
+      if (base + lane < st.logEnd) { const OpRec r = log[base + lane]; rk = r.key; rw = r.word; }
+      loaded = true;
+    }
+    const int h = pos - base;
+    const uint32_t hk = rlane(rk, h), hw = rlane(rw, h);
+    const int c = (int)(hk & 0xffu), nrec = (int)(hk >> 8);
+    // rows in the reference's order: the first two swap when the heap has row 1's node on top
+    const bool swap = (hw & kOpUnordered) && rlane(rh.n0, 1) != (hw & 0x3ffffffu);
+    const bool mine = lane > h && lane <= h + nrec;
+    const int myRow = (int)((rw >> 26) & 3u);
+    for (int i = 0; i < c; ++i) {
+      const int row = (swap && i < 2) ? 1 - i : i;
+      rh.pop(lane);
+      unsigned long long m = lanes_where(mine && myRow == row);
+      while (m) {
+        const int j = __ffsll((long long)m) - 1;
+        m &= m - 1;
+        const uint32_t key = rlane(rk, j), word = rlane(rw, j);
+        const uint32_t node = word & 0x3ffffffu;
+        // a node seen as open whose entry has left (its row came earlier in the pass) is pushed
+        int q = ((word >> 28) & 1u) ? rh.position(node, lane) : 0;
+        if (!q) {
+          if (rh.size >= kRegHeap) return false;
+          q = ++rh.size;
+        }
+        rh.bubble_up(q, key, node, lane);
+      }
+    }
+    pos += 1 + nrec;
+  }
+  st.synced = st.logEnd;
+  return true;
+}
+enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3, kAstarTie = 4, kAstarLogFull = 5 };
 
 BPSX_DEV float tri_area2d(const float* a, const float* b, const float* c) {
   const float abx = b[0] - a[0], abz = b[2] - a[2];
@@ -292,6 +423,8 @@ constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/
 #define BPSX_HASH 512
 #endif
 constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash table
+constexpr int kTagSlots = 128;
+constexpr int kRows = 4;                    // nodes expanded per pass of astar_fast, one per row of 16 lanes
 static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
 
 // LDS of one wavefront.
@@ -305,6 +438,7 @@ struct GeoLds {
   float w_total[kWindow];
   float w_cost[kWindow];
   float w_pos[3][kWindow];
+  uint32_t tag[kTagSlots];         // which nodes of a pass touch a polygon (see astar_fast)
 };
 // After A* its LDS is dead; the funnel reuses it for the corridor and its portals.  The
 // corridor is written while the nodes' links are still being read: it lies over the hash
@@ -329,6 +463,9 @@ struct GeoWave {
   int heapSize;
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
+  uint32_t tagNow;                   // mark of the current pass in L->tag, counting down
+  uint32_t exactRuns;                // queries run again with the exact heap
+  uint32_t tieReplays;               // ties resolved by replaying the operation log through the exact heap
 #ifdef BPSX_QUERY_TRACE
   uint32_t missTop, missNb, maxHeap;
 #endif
@@ -347,9 +484,16 @@ struct GeoWave {
   }
   // node i still has its position/cost/total in LDS
   BPSX_DEV bool in_window(int i) const { return i >= nodeCount - kWindow; }
-  static BPSX_DEV uint32_t hash(uint32_t ip) { return (__umul24(ip, 0x9e3779u) >> 9) & (kHashSize - 1); }
+  // the multiply as the full-rate 24-bit instruction (polygon indices have 15 bits)
+  static BPSX_DEV uint32_t hash(uint32_t ip) {
+    uint32_t m;
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(m) : "v"(ip), "s"(0x9e3779u));
+    return (m >> 9) & (kHashSize - 1);
+  }
   BPSX_DEV void clear() {
     for (int i = lane; i < kHashSize; i += 64) L->first[i] = (uint16_t)kChainEnd;
+    for (int i = lane; i < kTagSlots; i += 64) L->tag[i] = 0xffffffffu;
+    tagNow = 0x3fffffffu;
     heapSize = 0;
     nodeCount = 0;
     wave_sync();
@@ -613,18 +757,10 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     wave_sync();
     PHASE_MARK(5);
-    // ---- ordered phase, in edge order.  First the "nearest so far" record (lastBestNode of
-    // findPath): an update replaces it when its heuristic is lower; only lanes below the
-    // current record can matter, usually none.
+    // ---- ordered phase, in edge order: the open list.  (findPath's "nearest so far" record,
+    // lastBestNode, is not kept: it only matters to a search that ends without reaching the
+    // goal, and the caller reports DT_PARTIAL_RESULT as failure, PathFinder.cpp:506.)
     const uint32_t packed = (uint32_t)ni | (nb << 11);   // heap entry of this lane's node
-    unsigned long long better = lanes_where(update && heuristic < st.lastBestCost);
-    while (better) {
-      const int src = __ffsll((long long)better) - 1;
-      better &= better - 1;
-      const float h = lane_f(heuristic, src);
-      if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
-    }
-    // then the open list
     unsigned long long upd = lanes_where(update);
     const unsigned long long openMask = lanes_where(wasOpen);
     while (upd) {
@@ -819,16 +955,10 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     }
     wave_sync();
     PHASE_MARK(5);
-    // ---- ordered phase, in the reference's order: A's lanes come before B's.  First the
-    // "nearest so far" record (lastBestNode of findPath), then the open list.
+    // ---- ordered phase, in the reference's order: A's lanes come before B's.  (findPath's
+    // "nearest so far" record, lastBestNode, is not kept: it only matters to a search that ends
+    // without reaching the goal, which the caller reports as failure, PathFinder.cpp:506.)
     const uint32_t packed = (uint32_t)ni | (nb << 11);
-    unsigned long long better = lanes_where(update && heuristic < st.lastBestCost);
-    while (better) {
-      const int src = __ffsll((long long)better) - 1;
-      better &= better - 1;
-      const float h = lane_f(heuristic, src);
-      if (h < st.lastBestCost) { st.lastBestCost = h; st.lastBest = (int)(rlane(packed, src) & 0x7ffu); }
-    }
     const unsigned long long upd = lanes_where(update);
     const unsigned long long openMask = lanes_where(wasOpen);
     auto apply = [&](unsigned long long m) {
@@ -849,6 +979,242 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       apply(upd & ~0xffffull);
     }
     PHASE_MARK(6);
+  }
+  return kAstarEmpty;
+}
+
+// The expansion loop with the open list as a sorted array (OpenList), up to kRows nodes per
+// pass.  Row r of 16 lanes works on entry r of the list (lane 16 r + j on edge j of its
+// polygon): the edge records of all of them arrive in one load, and node lookup, costs, node
+// creation and stores are done by the same instructions for all rows.  Every row computes
+// from the state before the pass.  Rows 0 .. c-1 are what the reference does next, in that
+// order, when for every row j below c
+//   - entry j's total is below entry j + 1's, and every total that an earlier row puts on the
+//     open list is above it: entry j is then the only entry with the smallest total when its
+//     turn comes, whatever the arrangement of the reference's heap,
+//   - no earlier row creates or updates a node that row j reads (a neighbour of both, or row
+//     j's own node).  This is found with one LDS word per polygon hash: every lane that
+//     updates notes the pass and its row there (the earliest row wins), every lane then looks
+//     for a note of an earlier row.  Two polygons with the same hash only make c smaller.
+//   - entry j is not the goal (the goal ends the search when it is first in line).
+// The pass commits c >= 1 rows: their new nodes take consecutive indices in row and edge
+// order, their entries leave the list, their updates enter it.  A later row may improve the
+// node of an earlier one (it sees it as open, the reference as closed): both views lead to
+// the same node state and the same list, because a modify that finds no entry is a push.
+// Returns kAstarTie when the first two entries share the smallest total.
+template <bool S, bool W>
+BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops,
+                             bool frontResolved) {
+  const int lane = g.lane;
+  GeoLds* L = g.L;
+  const float H_SCALE = 0.999f;
+  const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
+  endIp = (uint32_t)uniform_i((int)endIp);
+  OpenList& ol = st.ol;
+  const int row = lane >> 4, el = lane & 15;
+  const bool edgeLane = el < kNvp;
+  const bool ownLane = el == kNvp;   // looks after the row's own node in the conflict test
+  constexpr unsigned long long kRowStart = 0x0001000100010001ull;
+  while (ol.size > 0) {
+    if (!S && g.nodeCount > kLinksLds - kRows * kNvp) return kAstarGrowLinks;
+#ifdef BPSX_BRIDGE_AT
+    if (ol.size > BPSX_BRIDGE_AT) return kAstarGrowHeap;   // test build: leave the sorted list early
+#endif
+    if (ol.size > (W ? 128 : 64) - kRows * kNvp) return kAstarGrowHeap;
+    if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
+    // ---- how many entries at the front are each the only one with their total
+    const unsigned long long uniq = lanes_where(ol.t0 < OpenList::down1(OpenList::kEmpty, ol.t0));
+    int lim = __builtin_ctzll(~uniq | (1ull << kRows));
+    bool pairTie = false;
+    if (frontResolved) { lim = 1; frontResolved = false; }   // the caller has put the reference's next node first
+    else if (lim == 0) {
+      // The first two entries share the smallest total.  When they are alone in that and their
+      // expansions are independent of each other (neither updates what the other reads, and
+      // whatever they put on the list lies above their total), the reference expands them one
+      // after the other, in the order its heap has them in, and ends in the same state either
+      // way: the pass takes both and notes in the log that their order is open.
+      if (!(uniq & 2ull)) return kAstarTie;
+      pairTie = true;
+      lim = __builtin_ctzll(~(uniq | 3ull) | (1ull << kRows));
+    }
+    const uint32_t cand = (uint32_t)__builtin_amdgcn_ds_bpermute(row * 4, (int)ol.n0);   // entry `row`
+    const int bi = (int)(cand & 0x7ffu);
+    const uint32_t ip = cand >> 11;
+    {
+      const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
+      if (goal & 1ull) {
+        const int biA = uniform_i(bi);
+        g.set_link<S>(biA, with_flags(g.link<S>(biA), 2u));
+        st.lastBest = biA;
+        return kAstarGoal;
+      }
+      if (goal) { const int jg = __builtin_ctzll(goal) >> 4; lim = jg < lim ? jg : lim; }
+      if (pairTie && lim < 2) return kAstarTie;   // the goal is one of the two
+    }
+    const bool rowOn = row < lim;
+    const bool act = edgeLane && rowOn;
+    uint32_t nb = kNoNb;
+    float m0 = 0, m1 = 0, m2 = 0;
+    if (act) {
+      const AEdge e = edges[ip * kNvp + (uint32_t)el];
+      nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
+    }
+    const int bis = rowOn ? bi : 0;
+    const uint32_t blink = g.link<S>(bis);
+    float b0, b1, b2, bcost;
+    uint32_t bparent;
+    {
+      const int w = bis & (kWindow - 1);
+      const bool binw = g.in_window(bis);
+      b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
+      bparent = L->w_parent[w];
+      if (lanes_where(!binw)) {
+        if (!binw) {
+          BPSX_KEEP_APART();
+          const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bis].pos);   // pos, cost
+          b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
+          bparent = g.ws->nodes[bis].parent;
+          BPSX_KEEP_APART();
+        }
+      }
+    }
+    // ---- node lookup; the row's own lane hashes its own polygon for the conflict test
+    const uint32_t bucket = GeoWave::hash(ownLane ? ip : nb);
+    uint32_t chainHead, hitLink;
+    int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
+    // the polygon the expanded node was reached from is not entered again
+    if (bparent && ni + 1 == (int)bparent) nb = kNoNb;
+    // ---- costs (new nodes have no index yet and read slot 0)
+    const bool valid = nb != kNoNb;
+    bool isNew = valid && ni < 0;
+    const int nis = (valid && !isNew) ? ni : 0;
+    const int rw = nis & (kWindow - 1);
+    uint32_t fl = link_flags(hitLink);
+    float p0 = L->w_pos[0][rw], p1 = L->w_pos[1][rw], p2 = L->w_pos[2][rw], oldTotal = L->w_total[rw];
+    const bool miss = valid && !isNew && !g.in_window(nis);
+    if (lanes_where(miss)) {
+      if (miss) {
+        const ANode& hn = g.ws->nodes[nis];
+        BPSX_KEEP_APART();
+        const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
+        p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = hn.total;
+        BPSX_KEEP_APART();
+      }
+    }
+    if (isNew) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }
+    const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
+    const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
+    const float cc = cx * cx + cy * cy + cz * cz, ee = ex * ex + ey * ey + ez * ez;
+    const float roots = sqrt_exact(lanes_up8(cc, ee));
+    const float curCost = roots * 1.0f;
+    const float toEnd = lanes_down8(roots);
+    const bool last = nb == endIp;
+    const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
+    const float heuristic = last ? 0.0f : toEnd * H_SCALE;
+    const float total = cost + heuristic;
+    const uint32_t tbits = __float_as_uint(total);
+    bool update = valid && !(fl && total >= oldTotal);
+    // ---- how many rows stand
+    int c = lim;
+    if (lim > 1) {
+      const uint32_t k1 = rlane(ol.t0, 1), k2 = rlane(ol.t0, 2), k3 = rlane(ol.t0, 3);
+      const unsigned long long v1 = lanes_where(update && tbits <= k1) & (pairTie ? 0xffffffffull : 0xffffull);   // both of a tied pair
+      const unsigned long long v2 = lanes_where(update && tbits <= k2) & 0xffffffffull;
+      const unsigned long long v3 = lanes_where(update && tbits <= k3) & 0xffffffffffffull;
+      const int jv = v1 ? 1 : (v2 ? 2 : (v3 ? 3 : 4));
+      c = jv < c ? jv : c;
+      // conflicts: the earliest row that updates a polygon leaves its mark, later rows look for it
+      g.tagNow--;
+      const uint32_t slot = bucket & (uint32_t)(kTagSlots - 1);
+      if (update) atomicMin(&L->tag[slot], (g.tagNow << 2) | (uint32_t)row);
+      wave_sync();
+      const bool reader = valid || (ownLane && rowOn);
+      const uint32_t seen = L->tag[reader ? slot : 0u];
+      const bool marked = reader && (seen >> 2) == g.tagNow;
+      const unsigned long long clash = lanes_where(marked && (int)(seen & 3u) < row);
+      if (clash) { const int jc = __builtin_ctzll(clash) >> 4; c = jc < c ? jc : c; }
+      if (pairTie) {
+        // rows 0 and 1 in either order: row 0 must not read what row 1 updates either
+        if (c < 2 || lanes_where(marked && row == 0 && (seen & 3u) == 1u)) return kAstarTie;
+      }
+    }
+    const bool rowIn = row < c;
+    update = update && rowIn;
+    isNew = isNew && rowIn;
+    const bool wasOpen = update && (fl & 1u) != 0;
+    (*pops) += (uint32_t)c;
+    // the committed rows' nodes are closed
+    if (el == 0 && rowIn) g.set_link<S>(bi, with_flags(blink, 2u));
+    // ---- new nodes take consecutive indices in row and edge order
+    {
+      const unsigned long long need = lanes_where(isNew);
+      if (need) {
+        const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
+        const int count = __popcll(need);
+        const int want = g.nodeCount + count;
+        // the reference carries on without the nodes that do not fit, but reports anything found
+        // after that as failure (only plain DT_SUCCESS counts, PathFinder.cpp:506): stop
+        if (S && want > kMaxNodes) { st.outOfNodes = true; return kAstarEmpty; }
+        if (isNew) ni = g.nodeCount + rank;
+        g.nodeCount = want;
+        bool pending = isNew;
+        uint32_t head = chainHead;
+        for (;;) {
+          if (pending) {
+            g.set_link<S>(ni, make_link(nb, 1u, head));
+            L->first[bucket] = (uint16_t)ni;
+          }
+          wave_sync();
+          if (count == 1) break;
+          if (pending) {
+            head = L->first[bucket];
+            pending = head != (uint32_t)ni;
+          }
+          wave_sync();
+          if (!lanes_where(pending)) break;
+        }
+      } else {
+        wave_sync();   // the closing writes above stay ahead of the link updates below
+      }
+    }
+    if (update) {
+      ANode& hn = g.ws->nodes[ni];
+      const int w = ni & (kWindow - 1);
+      const uint32_t parent = (uint32_t)bi + 1u;
+      if (!isNew) g.set_link<S>(ni, with_flags(hitLink, 1u));   // open (again)
+      if (g.in_window(ni)) {
+        L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2;
+        L->w_cost[w] = cost; L->w_total[w] = total;
+        L->w_parent[w] = (uint16_t)parent;
+      }
+      *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
+      *reinterpret_cast<uint2*>(&hn.total) = make_uint2(tbits, parent);
+    }
+    wave_sync();
+    // ---- the open list: the committed entries leave, the updates enter
+    ol.template drop_front<W>(c, lane);
+    const uint32_t packed = (uint32_t)ni | (nb << 11);
+    unsigned long long upd = lanes_where(update);
+    const unsigned long long openMask = lanes_where(wasOpen);
+    {
+      // the pass in the operation log: the header from an idle lane, the updates in lane order
+      const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(upd >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)upd, 0u));
+      const bool header = lane == 15;
+      const int nrec = __popcll(upd);
+      if (update || header) {
+        OpRec r;
+        r.key = header ? ((uint32_t)c | ((uint32_t)nrec << 8)) : tbits;
+        r.word = header ? (pairTie ? (kOpHeader | kOpUnordered | rlane(cand, 0)) : kOpHeader)
+                        : (packed | ((uint32_t)row << 26) | ((uint32_t)wasOpen << 28));
+        g.ws->oplog[st.logEnd + (header ? 0 : 1 + rank)] = r;
+      }
+      st.logEnd += 1 + nrec;
+    }
+    while (upd) {
+      const int src = __ffsll((long long)upd) - 1;
+      upd &= upd - 1;
+      ol.template update<W>((openMask >> src) & 1ull, rlane(packed, src), rlane(tbits, src), lane);
+    }
   }
   return kAstarEmpty;
 }
@@ -878,8 +1244,15 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #define ASTAR_ARGS g, st, edges, endIp, endPos, pops
 #endif
 #define ASTAR_RUN(M) astar_loop<M>(ASTAR_ARGS)
-  g.clear();
-  {
+  const uint32_t pops0 = *pops;
+  AstarExit ex;
+#ifdef BPSX_EXACT_ONLY
+  bool exact = true;
+#else
+  bool exact = false;   // first with the sorted open list; with the reference's heap when that meets a tie
+#endif
+  for (;;) {
+    g.clear();
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
     const float total = sqrtf(dx * dx + dy * dy + dz * dz) * 0.999f;
     g.nodeCount = 1;
@@ -896,46 +1269,104 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     }
     wave_sync();
     st.lastBest = 0;
-    st.lastBestCost = total;
     st.outOfNodes = false;
     st.rh.init(lane);
     st.rh.push(__float_as_uint(total), startIp << 11, lane);
-  }
-#ifdef BPSX_ONE_NODE_PER_PASS
-  AstarExit ex = ASTAR_RUN(0);
-  if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
-#else
-  // the loop is instantiated for links in LDS only or spilling, and for an open list within one
-  // register pair or two; a search moves on when one more pass could outgrow what it runs in
-  AstarExit ex;
-  bool spill = false, wide = false;
-  for (;;) {
-    if (!spill) ex = wide ? astar_loop2<false, true>(ASTAR_ARGS) : astar_loop2<false, false>(ASTAR_ARGS);
-    else ex = wide ? astar_loop2<true, true>(ASTAR_ARGS) : astar_loop2<true, false>(ASTAR_ARGS);
-    if (ex == kAstarGrowLinks) { g.linkSpills++; spill = true; }
-    else if (ex == kAstarGrowHeap && !wide) wide = true;
-    else break;
-  }
+    bool spill = false, wide = false;
+    if (!exact) {
+      st.ol.init();
+      st.ol.template update<false>(false, startIp << 11, __float_as_uint(total), lane);
+      st.logEnd = st.synced = 0;
+      // the loop is instantiated for links in LDS only or spilling, and for a list within one
+      // register pair or two; a search moves on when one more pass could outgrow what it runs in
+      bool resolved = false, restart = false;
+      for (;;) {
+        if (!spill) ex = wide ? astar_fast<false, true>(g, st, edges, endIp, endPos, pops, resolved) : astar_fast<false, false>(g, st, edges, endIp, endPos, pops, resolved);
+        else ex = wide ? astar_fast<true, true>(g, st, edges, endIp, endPos, pops, resolved) : astar_fast<true, false>(g, st, edges, endIp, endPos, pops, resolved);
+        resolved = false;
+        if (ex == kAstarGrowLinks) { g.linkSpills++; spill = true; continue; }
+        if (ex == kAstarGrowHeap && !wide) { wide = true; continue; }
+        if (ex != kAstarTie && ex != kAstarGrowHeap && ex != kAstarLogFull) break;
+        // the reference's heap is needed: bring it up to date from the log
+        if (!replay_log(g.ws->oplog, st, lane) || st.rh.size != st.ol.size) { restart = true; break; }
+#ifdef BPSX_VERIFY_REPLAY
+        {
+          // popping a copy of the rebuilt heap must give the list's entries in order
+          RegHeap copy = st.rh;
+          int badKey = 0, badNode = 0;
+          for (int i = 0; i < st.ol.size; ++i) {
+            const uint32_t hk = rlane(copy.t0, 1), hn = rlane(copy.n0, 1);
+            const uint32_t lk = i < 64 ? rlane(st.ol.t0, i) : rlane(st.ol.t1, i - 64), ln = i < 64 ? rlane(st.ol.n0, i) : rlane(st.ol.n1, i - 64);
+            if (hk != lk) badKey++;
+            else if (hn != ln) badNode++;
+            copy.pop(lane);
+          }
+          if (badKey) g.exactRuns += 1000000;
+          if (badNode) g.exactRuns += 1000;
+        }
 #endif
-  if (ex == kAstarGrowHeap) {
-    g.heapSpills++;
-    // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
-    const RegHeap& rh = st.rh;
-    auto put = [&](int i, uint32_t t, uint32_t n) {
-      const HeapEntry e{__uint_as_float(t), n & 0x7ffu};
-      if (i < kHeapLds) g.L->heap[i] = e;
-      else { BPSX_KEEP_APART(); g.ws->heap_spill[i] = e; BPSX_KEEP_APART(); }
-    };
-    if (lane >= 1 && lane <= rh.size) put(lane - 1, rh.t0, rh.n0);
-    if (64 + lane <= rh.size) put(63 + lane, rh.t1, rh.n1);
-    g.heapSize = rh.size;
-    wave_sync();
-    ex = ASTAR_RUN(2);
+        if (ex != kAstarTie) { g.heapSpills++; break; }   // the list or the log is full: on with the exact loops
+        // a tie: the reference pops what its heap has at the root.  That entry goes first.
+        g.tieReplays++;
+        const uint32_t root = rlane(st.rh.n0, 1);
+        const unsigned long long at = lanes_where(st.ol.n0 == root);
+        const int p = at ? __ffsll((long long)at) - 1 : -1;
+        if (p < 0 || rlane(st.ol.t0, p) != rlane(st.ol.t0, 0)) { restart = true; break; }
+        const uint32_t front = rlane(st.ol.n0, 0);
+        st.ol.n0 = wlane(st.ol.n0, root, 0);
+        st.ol.n0 = wlane(st.ol.n0, front, p);
+        resolved = true;
+      }
+      if (restart) {
+        // the heap outgrew the registers during the replay: the search runs again with the exact loops
+        g.exactRuns++;
+        *pops = pops0;
+        exact = true;
+        continue;
+      }
+      if (ex != kAstarGrowHeap && ex != kAstarLogFull) break;
+      // st.rh is the reference's heap as of now: the exact loops carry on from here
+    }
+#ifdef BPSX_ONE_NODE_PER_PASS
+    ex = ASTAR_RUN(0);
+    if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
+#else
+    {
+      wide = false;
+      for (;;) {
+        if (!spill) ex = wide ? astar_loop2<false, true>(ASTAR_ARGS) : astar_loop2<false, false>(ASTAR_ARGS);
+        else ex = wide ? astar_loop2<true, true>(ASTAR_ARGS) : astar_loop2<true, false>(ASTAR_ARGS);
+        if (ex == kAstarGrowLinks) { g.linkSpills++; spill = true; }
+        else if (ex == kAstarGrowHeap && !wide) wide = true;
+        else break;
+      }
+    }
+#endif
+    if (ex == kAstarGrowHeap) {
+      g.heapSpills++;
+      // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
+      const RegHeap& rh = st.rh;
+      auto put = [&](int i, uint32_t t, uint32_t n) {
+        const HeapEntry e{__uint_as_float(t), n & 0x7ffu};
+        if (i < kHeapLds) g.L->heap[i] = e;
+        else { BPSX_KEEP_APART(); g.ws->heap_spill[i] = e; BPSX_KEEP_APART(); }
+      };
+      if (lane >= 1 && lane <= rh.size) put(lane - 1, rh.t0, rh.n0);
+      if (64 + lane <= rh.size) put(63 + lane, rh.t1, rh.n1);
+      g.heapSize = rh.size;
+      wave_sync();
+      ex = ASTAR_RUN(2);
+    }
+    break;
   }
 #undef ASTAR_RUN
 #undef ASTAR_ARGS
-  (void)ex;
-  if (st.outOfNodes) return 0;   // no path to build: the result is a failure
+  // an open list that ran empty, or a pool that ran out, is DT_PARTIAL_RESULT or
+  // DT_OUT_OF_NODES in the reference: no path to build, the result is a failure
+#ifdef BPSX_DEBUG_BRIDGE
+  if (ex != kAstarGoal || st.outOfNodes) return -(1 + (int)ex + 10 * (int)st.outOfNodes + 100 * st.rh.size + 100000 * (int)(*pops - pops0));
+#endif
+  if (ex != kAstarGoal || st.outOfNodes) return 0;
   const int lastBest = st.lastBest;
   // getPathToNode: one walk up the parents notes the node indices (in the window's array of
   // positions, no longer needed), then all lanes fill the corridor, which overlays the hash heads;
@@ -1080,6 +1511,9 @@ BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q,
   unsigned long long phase_t0 = __builtin_readcyclecounter();
 #else
   const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops);
+#endif
+#ifdef BPSX_DEBUG_BRIDGE
+  if (n < 0) return (float)n;
 #endif
   if (n <= 0) return INF;
   *corridor += (uint32_t)n;

@@ -538,7 +538,7 @@ __global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* _
   for (int c = 0; c < kGeoClasses; ++c) first[c + 1] = first[c] + (uint32_t)uniform_i((int)counts[c]);
   const uint32_t nq = first[kGeoClasses], nlong = first[kLongClasses];
   GeoTotals T;
-  uint32_t linkSpills = 0, heapSpills = 0;
+  uint32_t linkSpills = 0, heapSpills = 0, exactRuns = 0, tieReplays = 0;
   if (threadIdx.x == 0) long_ticket = atomicAdd(head_long, 1u);
   __syncthreads();
   const uint32_t lt = (uint32_t)uniform_i((int)long_ticket);
@@ -550,12 +550,12 @@ __global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* _
     gl.ws = slot;
     gl.heapSize = 0;
     gl.nodeCount = 0;
-    gl.linkSpills = gl.heapSpills = 0;
+    gl.linkSpills = gl.heapSpills = gl.exactRuns = gl.tieReplays = 0;
     int cls = 0;
     while (lt >= first[cls + 1]) cls++;
     const GeoQuery q = queries[(size_t)cls * stride + (lt - first[cls])];
     serve_query(gl, nav, q, cls, out, last_cost, T);
-    linkSpills += gl.linkSpills; heapSpills += gl.heapSpills;
+    linkSpills += gl.linkSpills; heapSpills += gl.heapSpills; exactRuns += gl.exactRuns; tieReplays += gl.tieReplays;
     if (lane == 0) atomicAdd((unsigned long long*)&counters[kCntLongPath], 1ull);
   }
   geo::GeoWave g;
@@ -564,7 +564,7 @@ __global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* _
   g.ws = slot;
   g.heapSize = 0;
   g.nodeCount = 0;
-  g.linkSpills = g.heapSpills = 0;
+  g.linkSpills = g.heapSpills = g.exactRuns = g.tieReplays = 0;
   // tickets below `taken` went to the blocks' first wavefronts above
   const uint32_t taken = nlong < gridDim.x ? nlong : gridDim.x;
   for (;;) {
@@ -578,13 +578,15 @@ __global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* _
     const GeoQuery q = queries[(size_t)cls * stride + (qi - first[cls])];
     serve_query(g, nav, q, cls, out, last_cost, T);
   }
-  linkSpills += g.linkSpills; heapSpills += g.heapSpills;
+  linkSpills += g.linkSpills; heapSpills += g.heapSpills; exactRuns += g.exactRuns; tieReplays += g.tieReplays;
   if (lane == 0 && T.done) {
     atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)T.done);
     atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)T.pops);
     atomicAdd((unsigned long long*)&counters[kCntCorridor], (unsigned long long)T.corridor);
     if (linkSpills) atomicAdd((unsigned long long*)&counters[kCntLinkSpills], (unsigned long long)linkSpills);
     if (heapSpills) atomicAdd((unsigned long long*)&counters[kCntHeapSpills], (unsigned long long)heapSpills);
+    if (exactRuns) atomicAdd((unsigned long long*)&counters[kCntExactRuns], (unsigned long long)exactRuns);
+    if (tieReplays) atomicAdd((unsigned long long*)&counters[kCntTieReplays], (unsigned long long)tieReplays);
 #ifdef BPSX_PHASE_TIMING
     for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], T.phase_acc[k]);
 #endif

@@ -175,8 +175,11 @@ int bpsx_check_errors(bpsx_sim *sim);
  * more node links than the kernel keeps in LDS, [17] path searches whose open list outgrew
  * the kernel's registers (both continue in slower code; results are the same), [18] path
  * searches expected to be among the longest of their step, which the kernel runs with larger
- * LDS structures (same results). */
-#define BPSX_NUM_COUNTERS 19
+ * LDS structures (same results), [19] path searches run a second time with the reference's
+ * open-list arrangement throughout, [20] times two open nodes shared the smallest total and
+ * the reference's arrangement was rebuilt from the search's operation log to tell which comes
+ * first (same results either way). */
+#define BPSX_NUM_COUNTERS 21
 int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
 /* Per-kernel timing with HIP events on the step's own stream. While enabled, every
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
