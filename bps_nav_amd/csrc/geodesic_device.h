@@ -45,6 +45,11 @@ namespace bpsx {
 #else
 #define PHASE_MARK(k) do { } while (0)
 #endif
+#ifdef BPSX_ASM_MARKS
+#define FM(k) asm volatile("; FAST_MARK " #k)
+#else
+#define FM(k) do { } while (0)
+#endif
 
 BPSX_DEV void wave_sync() {
   // All lanes belong to one wavefront: LDS and memory operations issue in program order, so
@@ -289,7 +294,6 @@ struct OpenList {
   }
   // The first c entries leave (W false: the list lives in the first pair only).
   template <bool W> BPSX_DEV void drop_front(int c, int lane) {
-    size -= c;
     if (!W) {
       for (int i = 0; i < c; ++i) { t0 = down1(kEmpty, t0); n0 = down1(kNone, n0); }
     } else {
@@ -301,32 +305,38 @@ struct OpenList {
       t1 = same ? a1 : kEmpty; n1 = same ? b1 : kNone;
     }
   }
-  // push (open false) or modify (open true: the node's entry, if it still has one, leaves
-  // first) of node n with total t.  The entry goes behind those with totals up to t.
-  template <bool W> BPSX_DEV void update(bool open, uint32_t n, uint32_t t, int lane) {
-    unsigned long long m0 = lanes_where(t0 > t), m1 = W ? lanes_where(t1 > t) : 0ull;
-    int r = -1;
-    if (open) {
-      const unsigned long long h0 = lanes_where(n0 == n);
-      if (h0) r = __ffsll((long long)h0) - 1;
-      else if (W) { const unsigned long long h1 = lanes_where(n1 == n); if (h1) r = 64 + __ffsll((long long)h1) - 1; }
+  // the number of entries, after drops and updates (which do not keep it)
+  template <bool W> BPSX_DEV void count() {
+    size = __popcll(lanes_where(t0 != kEmpty));
+    if (W) size += __popcll(lanes_where(t1 != kEmpty));
+  }
+  // lane L takes v of lane L - 1 (lane 0: anything)
+  static BPSX_DEV uint32_t from_below(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, true);
+  }
+  // Node n gets total t: its entry, if it has one, leaves, and the new entry goes behind those
+  // with totals up to t.  (A node has an entry exactly when it is open and has not just been
+  // taken off the front, so whether this is the reference's push or its modify need not be told.)
+  // No branches: without an old entry the "entries up to the old place" are all entries.
+  template <bool W> BPSX_DEV void update(uint32_t n, uint32_t t) {
+    const unsigned long long g0 = lanes_where(t0 > t), h0 = lanes_where(n0 == n);
+    if (!W) {
+      // an empty mask gives -1: the shift count 63 then keeps every lane
+      const unsigned long long m0 = g0 & ((2ull << ((__ffsll((long long)h0) - 1) & 63)) - 1ull);
+      const int p = __ffsll((long long)m0) - 1;
+      t0 = wlane(pick(m0, from_below(t0), t0), t, p);
+      n0 = wlane(pick(m0, from_below(n0), n0), n, p);
+      return;
     }
-    if (r >= 0) {
-      // only the entries from the new place up to the old one move
-      if (r < 64) { m0 &= (2ull << r) - 1ull; m1 = 0; }
-      else m1 &= (2ull << (r - 64)) - 1ull;
-    } else {
-      size++;
-    }
+    const unsigned long long g1 = lanes_where(t1 > t), h1 = lanes_where(n1 == n);
+    unsigned long long m0 = g0, m1 = g1;
+    if (h0) { m0 &= (2ull << (__ffsll((long long)h0) - 1)) - 1ull; m1 = 0; }
+    else if (h1) m1 &= (2ull << (__ffsll((long long)h1) - 1)) - 1ull;
     const int p = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
-    if (W) {
-      const uint32_t ct = rlane(t0, 63), cn = rlane(n0, 63);   // what moves up into the second pair
-      const uint32_t s1 = up1(ct, t1), u1 = up1(cn, n1);
-      t1 = pick(m1, s1, t1); n1 = pick(m1, u1, n1);
-    }
-    const uint32_t s0 = up1(t0, t0), u0 = up1(n0, n0);
-    t0 = pick(m0, s0, t0); n0 = pick(m0, u0, n0);
-    if (!W || p < 64) { t0 = wlane(t0, t, p); n0 = wlane(n0, n, p); }
+    const uint32_t ct = rlane(t0, 63), cn = rlane(n0, 63);   // what moves up into the second pair
+    t1 = pick(m1, up1(ct, t1), t1); n1 = pick(m1, up1(cn, n1), n1);
+    t0 = pick(m0, from_below(t0), t0); n0 = pick(m0, from_below(n0), n0);
+    if (p < 64) { t0 = wlane(t0, t, p); n0 = wlane(n0, n, p); }
     else { t1 = wlane(t1, t, p - 64); n1 = wlane(n1, n, p - 64); }
   }
 };
@@ -1015,33 +1025,41 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const bool edgeLane = el < kNvp;
   const bool ownLane = el == kNvp;   // looks after the row's own node in the conflict test
   constexpr unsigned long long kRowStart = 0x0001000100010001ull;
-  while (ol.size > 0) {
+  constexpr unsigned long long kRows1 = 0xffffull, kRows2 = 0xffffffffull, kRows3 = 0xffffffffffffull;   // lanes of the first rows
+  // Written for few instructions on the common path: what is rare sits behind one branch each,
+  // and conditions that feed a ballot are folded into the compared value first, so that the
+  // ballot is the comparison's own result.
+  for (;;) {
+    if (ol.size <= 0) return kAstarEmpty;
     if (!S && g.nodeCount > kLinksLds - kRows * kNvp) return kAstarGrowLinks;
 #ifdef BPSX_BRIDGE_AT
     if (ol.size > BPSX_BRIDGE_AT) return kAstarGrowHeap;   // test build: leave the sorted list early
 #endif
     if (ol.size > (W ? 128 : 64) - kRows * kNvp) return kAstarGrowHeap;
     if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
+    FM(0);
     // ---- how many entries at the front are each the only one with their total
     const unsigned long long uniq = lanes_where(ol.t0 < OpenList::down1(OpenList::kEmpty, ol.t0));
     int lim = __builtin_ctzll(~uniq | (1ull << kRows));
-    bool pairTie = false;
-    if (frontResolved) { lim = 1; frontResolved = false; }   // the caller has put the reference's next node first
-    else if (lim == 0) {
-      // The first two entries share the smallest total.  When they are alone in that and their
-      // expansions are independent of each other (neither updates what the other reads, and
-      // whatever they put on the list lies above their total), the reference expands them one
-      // after the other, in the order its heap has them in, and ends in the same state either
-      // way: the pass takes both and notes in the log that their order is open.
-      if (!(uniq & 2ull)) return kAstarTie;
-      pairTie = true;
-      lim = __builtin_ctzll(~(uniq | 3ull) | (1ull << kRows));
-    }
     const uint32_t cand = (uint32_t)__builtin_amdgcn_ds_bpermute(row * 4, (int)ol.n0);   // entry `row`
     const int bi = (int)(cand & 0x7ffu);
     const uint32_t ip = cand >> 11;
-    {
-      const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
+    const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
+    bool pairTie = false;
+    unsigned long long rowsAt1 = kRows1;   // rows whose updates must lie above entry 1's total
+    if (__builtin_expect(frontResolved || lim == 0 || goal != 0, 0)) {
+      if (frontResolved) { lim = 1; frontResolved = false; }   // the caller has put the reference's next node first
+      else if (lim == 0) {
+        // The first two entries share the smallest total.  When they are alone in that and their
+        // expansions are independent of each other (neither updates what the other reads, and
+        // whatever they put on the list lies above their total), the reference expands them one
+        // after the other, in the order its heap has them in, and ends in the same state either
+        // way: the pass takes both and notes in the log that their order is open.
+        if (!(uniq & 2ull)) return kAstarTie;
+        pairTie = true;
+        rowsAt1 = kRows2;
+        lim = __builtin_ctzll(~(uniq | 3ull) | (1ull << kRows));
+      }
       if (goal & 1ull) {
         const int biA = uniform_i(bi);
         g.set_link<S>(biA, with_flags(g.link<S>(biA), 2u));
@@ -1051,6 +1069,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       if (goal) { const int jg = __builtin_ctzll(goal) >> 4; lim = jg < lim ? jg : lim; }
       if (pairTie && lim < 2) return kAstarTie;   // the goal is one of the two
     }
+    FM(1);
     const bool rowOn = row < lim;
     const bool act = edgeLane && rowOn;
     uint32_t nb = kNoNb;
@@ -1065,11 +1084,11 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     uint32_t bparent;
     {
       const int w = bis & (kWindow - 1);
-      const bool binw = g.in_window(bis);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
       bparent = L->w_parent[w];
-      if (lanes_where(!binw)) {
-        if (!binw) {
+      const bool bout = bis < g.nodeCount - kWindow;
+      if (lanes_where(bout)) {
+        if (bout) {
           BPSX_KEEP_APART();
           const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bis].pos);   // pos, cost
           b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
@@ -1078,20 +1097,21 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         }
       }
     }
+    FM(2);
     // ---- node lookup; the row's own lane hashes its own polygon for the conflict test
     const uint32_t bucket = GeoWave::hash(ownLane ? ip : nb);
     uint32_t chainHead, hitLink;
     int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
     // the polygon the expanded node was reached from is not entered again
     if (bparent && ni + 1 == (int)bparent) nb = kNoNb;
-    // ---- costs (new nodes have no index yet and read slot 0)
+    FM(3);
+    // ---- costs.  A lane without a node to read (idle, or its node is new) reads window slot 127.
     const bool valid = nb != kNoNb;
-    bool isNew = valid && ni < 0;
-    const int nis = (valid && !isNew) ? ni : 0;
+    const int nis = (valid && ni >= 0) ? ni : 0x7fffffff;
     const int rw = nis & (kWindow - 1);
     uint32_t fl = link_flags(hitLink);
     float p0 = L->w_pos[0][rw], p1 = L->w_pos[1][rw], p2 = L->w_pos[2][rw], oldTotal = L->w_total[rw];
-    const bool miss = valid && !isNew && !g.in_window(nis);
+    const bool miss = nis < g.nodeCount - kWindow;
     if (lanes_where(miss)) {
       if (miss) {
         const ANode& hn = g.ws->nodes[nis];
@@ -1101,7 +1121,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         BPSX_KEEP_APART();
       }
     }
-    if (isNew) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }
+    if (ni < 0) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }   // a new node lies on the portal's midpoint
     const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
     const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
     const float cc = cx * cx + cy * cy + cz * cz, ee = ex * ex + ey * ey + ez * ez;
@@ -1112,42 +1132,46 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
     const float heuristic = last ? 0.0f : toEnd * H_SCALE;
     const float total = cost + heuristic;
-    const uint32_t tbits = __float_as_uint(total);
-    bool update = valid && !(fl && total >= oldTotal);
+    // the total as bits where the lane updates its node, all ones where it does not
+    uint32_t tb = (valid && !(fl && total >= oldTotal)) ? __float_as_uint(total) : 0xffffffffu;
+    FM(4);
     // ---- how many rows stand
     int c = lim;
     if (lim > 1) {
       const uint32_t k1 = rlane(ol.t0, 1), k2 = rlane(ol.t0, 2), k3 = rlane(ol.t0, 3);
-      const unsigned long long v1 = lanes_where(update && tbits <= k1) & (pairTie ? 0xffffffffull : 0xffffull);   // both of a tied pair
-      const unsigned long long v2 = lanes_where(update && tbits <= k2) & 0xffffffffull;
-      const unsigned long long v3 = lanes_where(update && tbits <= k3) & 0xffffffffffffull;
+      const unsigned long long v1 = lanes_where(tb <= k1) & rowsAt1;
+      const unsigned long long v2 = lanes_where(tb <= k2) & kRows2;
+      const unsigned long long v3 = lanes_where(tb <= k3) & kRows3;
       const int jv = v1 ? 1 : (v2 ? 2 : (v3 ? 3 : 4));
       c = jv < c ? jv : c;
-      // conflicts: the earliest row that updates a polygon leaves its mark, later rows look for it
+      // conflicts: the earliest row that updates a polygon leaves its mark (pass, row) at the
+      // polygon's hash, later rows look for it: a mark of this pass is base + row
       g.tagNow--;
+      const uint32_t base = g.tagNow << 2;
       const uint32_t slot = bucket & (uint32_t)(kTagSlots - 1);
-      if (update) atomicMin(&L->tag[slot], (g.tagNow << 2) | (uint32_t)row);
+      if (tb != 0xffffffffu) atomicMin(&L->tag[slot], base | (uint32_t)row);
       wave_sync();
-      const bool reader = valid || (ownLane && rowOn);
-      const uint32_t seen = L->tag[reader ? slot : 0u];
-      const bool marked = reader && (seen >> 2) == g.tagNow;
-      const unsigned long long clash = lanes_where(marked && (int)(seen & 3u) < row);
+      const uint32_t seen = L->tag[slot] - base;   // the marking row, or something above 3
+      const uint32_t seenr = (valid || (ownLane && rowOn)) ? seen : 0xffffffffu;
+      const unsigned long long clash = lanes_where(seenr < (uint32_t)row);
       if (clash) { const int jc = __builtin_ctzll(clash) >> 4; c = jc < c ? jc : c; }
-      if (pairTie) {
+      if (__builtin_expect(pairTie, 0)) {
         // rows 0 and 1 in either order: row 0 must not read what row 1 updates either
-        if (c < 2 || lanes_where(marked && row == 0 && (seen & 3u) == 1u)) return kAstarTie;
+        if (c < 2 || (lanes_where(seenr == 1u) & kRows1)) return kAstarTie;
       }
     }
+    FM(5);
     const bool rowIn = row < c;
-    update = update && rowIn;
-    isNew = isNew && rowIn;
-    const bool wasOpen = update && (fl & 1u) != 0;
+    tb = rowIn ? tb : 0xffffffffu;
+    const bool update = tb != 0xffffffffu;
+    const bool isNew = update && ni < 0;   // a new node is always taken
     (*pops) += (uint32_t)c;
     // the committed rows' nodes are closed
     if (el == 0 && rowIn) g.set_link<S>(bi, with_flags(blink, 2u));
+    FM(6);
     // ---- new nodes take consecutive indices in row and edge order
     {
-      const unsigned long long need = lanes_where(isNew);
+      const unsigned long long need = lanes_where((update ? ni : 0) < 0);
       if (need) {
         const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
         const int count = __popcll(need);
@@ -1177,6 +1201,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         wave_sync();   // the closing writes above stay ahead of the link updates below
       }
     }
+    FM(7);
     if (update) {
       ANode& hn = g.ws->nodes[ni];
       const int w = ni & (kWindow - 1);
@@ -1188,14 +1213,14 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         L->w_parent[w] = (uint16_t)parent;
       }
       *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
-      *reinterpret_cast<uint2*>(&hn.total) = make_uint2(tbits, parent);
+      *reinterpret_cast<uint2*>(&hn.total) = make_uint2(tb, parent);
     }
     wave_sync();
+    FM(8);
     // ---- the open list: the committed entries leave, the updates enter
     ol.template drop_front<W>(c, lane);
     const uint32_t packed = (uint32_t)ni | (nb << 11);
-    unsigned long long upd = lanes_where(update);
-    const unsigned long long openMask = lanes_where(wasOpen);
+    unsigned long long upd = lanes_where(tb != 0xffffffffu);
     {
       // the pass in the operation log: the header from an idle lane, the updates in lane order
       const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(upd >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)upd, 0u));
@@ -1203,20 +1228,22 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const int nrec = __popcll(upd);
       if (update || header) {
         OpRec r;
-        r.key = header ? ((uint32_t)c | ((uint32_t)nrec << 8)) : tbits;
+        r.key = header ? ((uint32_t)c | ((uint32_t)nrec << 8)) : tb;
         r.word = header ? (pairTie ? (kOpHeader | kOpUnordered | rlane(cand, 0)) : kOpHeader)
-                        : (packed | ((uint32_t)row << 26) | ((uint32_t)wasOpen << 28));
+                        : (packed | ((uint32_t)row << 26) | ((fl & 1u) << 28));
         g.ws->oplog[st.logEnd + (header ? 0 : 1 + rank)] = r;
       }
       st.logEnd += 1 + nrec;
     }
+    FM(9);
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
-      ol.template update<W>((openMask >> src) & 1ull, rlane(packed, src), rlane(tbits, src), lane);
+      ol.template update<W>(rlane(packed, src), rlane(tb, src));
     }
+    ol.template count<W>();
+    FM(10);
   }
-  return kAstarEmpty;
 }
 
 // Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
@@ -1275,7 +1302,8 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     bool spill = false, wide = false;
     if (!exact) {
       st.ol.init();
-      st.ol.template update<false>(false, startIp << 11, __float_as_uint(total), lane);
+      st.ol.template update<false>(startIp << 11, __float_as_uint(total));
+      st.ol.template count<false>();
       st.logEnd = st.synced = 0;
       // the loop is instantiated for links in LDS only or spilling, and for a list within one
       // register pair or two; a search moves on when one more pass could outgrow what it runs in

@@ -523,7 +523,7 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
 // the whole block's LDS (the larger instantiation: no link spills, half the window misses,
 // shorter hash chains; 7 % faster on such searches) while its second wavefront leaves.
 constexpr int kLongClasses = 2;   // expected cost of 1400 nodes and more
-__global__ __launch_bounds__(128) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
                                                   const uint32_t* __restrict__ counts, uint32_t* head, uint32_t* head_long,
                                                   float* out, uint32_t* last_cost, GeoSlot* slots, uint64_t* counters) {
   constexpr size_t kHalf = sizeof(geo::GeoShared);
