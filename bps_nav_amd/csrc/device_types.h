@@ -47,6 +47,7 @@ struct AEdge {
                  // a polygon that passes the query filter), else kNoNb
 };
 static_assert(sizeof(AEdge) == 16, "AEdge");
+constexpr int kEdgeStride = 8;   // records per polygon in HBM: six edges and two unused, one 128-byte line
 constexpr uint32_t kNoNb = 0xffffu;
 
 // dtBVNode repacked at upload: same quantised bounds; a leaf carries its polygon index, an
@@ -114,7 +115,7 @@ constexpr uint32_t kAgentDone = 1u, kAgentMoved = 2u, kAgentReuse = 4u, kAgentSk
 
 struct NavData {
   const PolyRec* polys;
-  const AEdge* aedges;     // [polygon][kNvp]
+  const AEdge* aedges;     // [polygon][kEdgeStride]
   const BVNodeDev* bv;
   const uint8_t* dtris;    // [.][4]
   const float* dverts;     // [.][3]

@@ -305,7 +305,7 @@ static int upload_scene(bpsx_sim* sim, HostScene& s, uint32_t entry, hipStream_t
   sim->ranges[entry] = r;
   const auto H2D = hipMemcpyHostToDevice;
   HIP_TRY(hipMemcpyAsync(sim->d_polys + r.poly, s.polys.data(), r.npoly * sizeof(PolyRec), H2D, st));
-  HIP_TRY(hipMemcpyAsync(sim->d_aedges + r.poly * kNvp, s.aedges.data(), s.aedges.size() * sizeof(AEdge), H2D, st));
+  HIP_TRY(hipMemcpyAsync(sim->d_aedges + r.poly * kEdgeStride, s.aedges.data(), s.aedges.size() * sizeof(AEdge), H2D, st));
   if (r.nbv) HIP_TRY(hipMemcpyAsync(sim->d_bv + r.bv, s.bv.data(), r.nbv * sizeof(BVNodeDev), H2D, st));
   if (r.ntri) HIP_TRY(hipMemcpyAsync(sim->d_dtris + r.tri * 4, s.dtris.data(), s.dtris.size(), H2D, st));
   if (r.ndv) HIP_TRY(hipMemcpyAsync(sim->d_dverts + r.dv * 3, s.dverts.data(), s.dverts.size() * 4, H2D, st));
@@ -460,7 +460,7 @@ int bpsx_finalize(bpsx_sim* sim) {
   if (cpoly > 0xfffffff0ull || ctri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
   int rc;
   if ((rc = sim->alloc(&sim->d_polys, cpoly))) return rc;
-  if ((rc = sim->alloc(&sim->d_aedges, cpoly * kNvp))) return rc;
+  if ((rc = sim->alloc(&sim->d_aedges, cpoly * kEdgeStride))) return rc;
   if ((rc = sim->alloc(&sim->d_bv, cbv))) return rc;
   if ((rc = sim->alloc(&sim->d_dtris, ctri * 4))) return rc;
   if ((rc = sim->alloc(&sim->d_dverts, cdv * 3))) return rc;

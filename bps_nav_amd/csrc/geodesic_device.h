@@ -47,6 +47,11 @@ namespace bpsx {
 #endif
 #ifdef BPSX_ASM_MARKS
 #define FM(k) asm volatile("; FAST_MARK " #k)
+#elif defined(BPSX_PHASE_TIMING)
+// marks of the sorted-list loop -> counters: 0 front of the list, 1 fetch, 2 lookup, 3 costs, 4 rows that stand,
+// 5 closing, new nodes and stores, 6 list and log; 7 counts the passes
+#define FM(k) do { constexpr int slot_[11] = {7, 0, 1, 2, 3, 4, 5, 5, 5, 6, 6}; const unsigned long long now_ = __builtin_readcyclecounter(); \
+    if ((k) == 0) g.phase[7]++; else g.phase[slot_[k]] += now_ - g.phase_t0; g.phase_t0 = now_; } while (0)
 #else
 #define FM(k) do { } while (0)
 #endif
@@ -80,6 +85,22 @@ BPSX_DEV uint32_t wlane(uint32_t old, uint32_t v, int lane) {
   const int sv = __builtin_amdgcn_readfirstlane((int)v), sl = __builtin_amdgcn_readfirstlane(lane);
   asm("s_mov_b32 m0, %2\n\tv_writelane_b32 %0, %1, m0" : "+v"(old) : "s"(sv), "s"(sl) : "m0");
   return old;
+}
+
+// index of the lowest set bit, -1 for an empty mask (the instruction's own convention)
+BPSX_DEV int first_lane(unsigned long long mask) {
+  int r;
+  asm("s_ff1_i32_b64 %0, %1" : "=s"(r) : "s"(mask));
+  return r;
+}
+BPSX_DEV unsigned long long without_lane(unsigned long long mask, int lane) {
+  asm("s_bitset0_b64 %0, %1" : "+s"(mask) : "s"(lane));
+  return mask;
+}
+// a and b with lane `lane` replaced by va and vb (all three uniform): one M0 write for both
+BPSX_DEV void wlane2(uint32_t& a, uint32_t va, uint32_t& b, uint32_t vb, int lane) {
+  const int sa = __builtin_amdgcn_readfirstlane((int)va), sb = __builtin_amdgcn_readfirstlane((int)vb), sl = __builtin_amdgcn_readfirstlane(lane);
+  asm("s_mov_b32 m0, %4\n\tv_writelane_b32 %0, %2, m0\n\tv_writelane_b32 %1, %3, m0" : "+v"(a), "+v"(b) : "s"(sa), "s"(sb), "s"(sl) : "m0");
 }
 
 // lanes 8..15 of each row of 16 take src of the lane 8 below them, lanes 0..7 keep low
@@ -318,14 +339,15 @@ struct OpenList {
   // with totals up to t.  (A node has an entry exactly when it is open and has not just been
   // taken off the front, so whether this is the reference's push or its modify need not be told.)
   // No branches: without an old entry the "entries up to the old place" are all entries.
-  template <bool W> BPSX_DEV void update(uint32_t n, uint32_t t) {
+  template <bool W> BPSX_DEV void update(uint32_t n, uint32_t t, int lane) {
     const unsigned long long g0 = lanes_where(t0 > t), h0 = lanes_where(n0 == n);
     if (!W) {
-      // an empty mask gives -1: the shift count 63 then keeps every lane
-      const unsigned long long m0 = g0 & ((2ull << ((__ffsll((long long)h0) - 1) & 63)) - 1ull);
-      const int p = __ffsll((long long)m0) - 1;
-      t0 = wlane(pick(m0, from_below(t0), t0), t, p);
-      n0 = wlane(pick(m0, from_below(n0), n0), n, p);
+      // without an old entry its place is -1: as an unsigned bound that keeps every lane
+      const unsigned long long m0 = g0 & lanes_where((uint32_t)lane <= (uint32_t)first_lane(h0));
+      const int p = first_lane(m0);   // never empty: the unused places compare greater
+      t0 = pick(m0, from_below(t0), t0);
+      n0 = pick(m0, from_below(n0), n0);
+      wlane2(t0, t, n0, n, p);
       return;
     }
     const unsigned long long g1 = lanes_where(t1 > t), h1 = lanes_where(n1 == n);
@@ -418,7 +440,7 @@ namespace bpsx {
 namespace BPSX_GEO_NS {
 
 #ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 1152
+#define BPSX_LINKS_LDS 1144
 #endif
 #ifndef BPSX_HEAP_LDS
 #define BPSX_HEAP_LDS 32
@@ -474,6 +496,9 @@ struct GeoWave {
   int nodeCount;
   uint32_t linkSpills, heapSpills;   // queries that left the LDS links / the register heap
   uint32_t tagNow;                   // mark of the current pass in L->tag, counting down
+#ifdef BPSX_PHASE_TIMING
+  unsigned long long phase[8], phase_t0;
+#endif
   uint32_t exactRuns;                // queries run again with the exact heap
   uint32_t tieReplays;               // ties resolved by replaying the operation log through the exact heap
 #ifdef BPSX_QUERY_TRACE
@@ -641,7 +666,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
     if (lane < kNvp) {
-      const AEdge e = edges[bestIp * kNvp + lane];
+      const AEdge e = edges[bestIp * kEdgeStride + lane];
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
     float b0, b1, b2, bcost;
@@ -841,7 +866,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
     if (act) {
-      const AEdge e = edges[(rowB ? ipB : ipA) * kNvp + (uint32_t)el];
+      const AEdge e = edges[(rowB ? ipB : ipA) * kEdgeStride + (uint32_t)el];
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
     float b0, b1, b2, bcost;
@@ -1026,6 +1051,8 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const bool ownLane = el == kNvp;   // looks after the row's own node in the conflict test
   constexpr unsigned long long kRowStart = 0x0001000100010001ull;
   constexpr unsigned long long kRows1 = 0xffffull, kRows2 = 0xffffffffull, kRows3 = 0xffffffffffffull;   // lanes of the first rows
+  unsigned long long resolved = frontResolved ? 1ull : 0ull;
+  uint32_t warm = 0;   // see the prefetch below
   // Written for few instructions on the common path: what is rare sits behind one branch each,
   // and conditions that feed a ballot are folded into the compared value first, so that the
   // ballot is the comparison's own result.
@@ -1047,8 +1074,8 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
     bool pairTie = false;
     unsigned long long rowsAt1 = kRows1;   // rows whose updates must lie above entry 1's total
-    if (__builtin_expect(frontResolved || lim == 0 || goal != 0, 0)) {
-      if (frontResolved) { lim = 1; frontResolved = false; }   // the caller has put the reference's next node first
+    if (__builtin_expect((goal | ((uniq & 1ull) ^ 1ull) | resolved) != 0, 0)) {
+      if (resolved) { lim = 1; resolved = 0; }   // the caller has put the reference's next node first
       else if (lim == 0) {
         // The first two entries share the smallest total.  When they are alone in that and their
         // expansions are independent of each other (neither updates what the other reads, and
@@ -1075,9 +1102,10 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
     if (act) {
-      const AEdge e = edges[ip * kNvp + (uint32_t)el];
+      const AEdge e = edges[ip * kEdgeStride + (uint32_t)el];
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
+    asm volatile("" ::"v"(warm));   // the previous pass's prefetch has a consumer: here, where the pass waits for memory anyway
     const int bis = rowOn ? bi : 0;
     const uint32_t blink = g.link<S>(bis);
     float b0, b1, b2, bcost;
@@ -1086,15 +1114,12 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const int w = bis & (kWindow - 1);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
       bparent = L->w_parent[w];
-      const bool bout = bis < g.nodeCount - kWindow;
-      if (lanes_where(bout)) {
-        if (bout) {
-          BPSX_KEEP_APART();
-          const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bis].pos);   // pos, cost
-          b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
-          bparent = g.ws->nodes[bis].parent;
-          BPSX_KEEP_APART();
-        }
+      if (bis < g.nodeCount - kWindow) {   // the node has left the window: rare
+        BPSX_KEEP_APART();
+        const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bis].pos);   // pos, cost
+        b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
+        bparent = g.ws->nodes[bis].parent;
+        BPSX_KEEP_APART();
       }
     }
     FM(2);
@@ -1111,15 +1136,12 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const int rw = nis & (kWindow - 1);
     uint32_t fl = link_flags(hitLink);
     float p0 = L->w_pos[0][rw], p1 = L->w_pos[1][rw], p2 = L->w_pos[2][rw], oldTotal = L->w_total[rw];
-    const bool miss = nis < g.nodeCount - kWindow;
-    if (lanes_where(miss)) {
-      if (miss) {
-        const ANode& hn = g.ws->nodes[nis];
-        BPSX_KEEP_APART();
-        const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
-        p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = hn.total;
-        BPSX_KEEP_APART();
-      }
+    if (nis < g.nodeCount - kWindow) {   // the node has left the window: rare
+      const ANode& hn = g.ws->nodes[nis];
+      BPSX_KEEP_APART();
+      const float4 pc = *reinterpret_cast<const float4*>(hn.pos);     // pos, cost
+      p0 = pc.x; p1 = pc.y; p2 = pc.z; oldTotal = hn.total;
+      BPSX_KEEP_APART();
     }
     if (ni < 0) { p0 = m0; p1 = m1; p2 = m2; fl = 0; }   // a new node lies on the portal's midpoint
     const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
@@ -1137,6 +1159,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     FM(4);
     // ---- how many rows stand
     int c = lim;
+    bool pairFails = false;
     if (lim > 1) {
       const uint32_t k1 = rlane(ol.t0, 1), k2 = rlane(ol.t0, 2), k3 = rlane(ol.t0, 3);
       const unsigned long long v1 = lanes_where(tb <= k1) & rowsAt1;
@@ -1153,13 +1176,12 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       wave_sync();
       const uint32_t seen = L->tag[slot] - base;   // the marking row, or something above 3
       const uint32_t seenr = (valid || (ownLane && rowOn)) ? seen : 0xffffffffu;
-      const unsigned long long clash = lanes_where(seenr < (uint32_t)row);
-      if (clash) { const int jc = __builtin_ctzll(clash) >> 4; c = jc < c ? jc : c; }
-      if (__builtin_expect(pairTie, 0)) {
-        // rows 0 and 1 in either order: row 0 must not read what row 1 updates either
-        if (c < 2 || (lanes_where(seenr == 1u) & kRows1)) return kAstarTie;
-      }
+      const uint32_t jc = (uint32_t)first_lane(lanes_where(seenr < (uint32_t)row)) >> 4;   // none: far above 4
+      c = jc < (uint32_t)c ? (int)jc : c;
+      // rows 0 and 1 of a tied pair in either order: row 0 must not read what row 1 updates either
+      if (__builtin_expect(pairTie, 0)) pairFails = c < 2 || (lanes_where(seenr == 1u) & kRows1) != 0;
     }
+    if (__builtin_expect(pairFails, 0)) return kAstarTie;
     FM(5);
     const bool rowIn = row < c;
     tb = rowIn ? tb : 0xffffffffu;
@@ -1168,6 +1190,10 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     (*pops) += (uint32_t)c;
     // the committed rows' nodes are closed
     if (el == 0 && rowIn) g.set_link<S>(bi, with_flags(blink, 2u));
+    // The edge records of a polygon that enters the open list are asked for now: the scenes'
+    // records are far larger than the caches, and a node is expanded one pass later at the
+    // earliest, by which time its line (one per polygon) has arrived in L2.
+    if (update) warm = edges[nb * kEdgeStride].nb;
     FM(6);
     // ---- new nodes take consecutive indices in row and edge order
     {
@@ -1237,9 +1263,9 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     }
     FM(9);
     while (upd) {
-      const int src = __ffsll((long long)upd) - 1;
-      upd &= upd - 1;
-      ol.template update<W>(rlane(packed, src), rlane(tb, src));
+      const int src = first_lane(upd);
+      upd = without_lane(upd, src);
+      ol.template update<W>(rlane(packed, src), rlane(tb, src), lane);
     }
     ol.template count<W>();
     FM(10);
@@ -1264,7 +1290,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     return 1;
   }
   AstarState st;
-  const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kNvp;
+  const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kEdgeStride;
 #ifdef BPSX_PHASE_TIMING
 #define ASTAR_ARGS g, st, edges, endIp, endPos, pops, phase_acc, phase_t0
 #else
@@ -1301,8 +1327,12 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     st.rh.push(__float_as_uint(total), startIp << 11, lane);
     bool spill = false, wide = false;
     if (!exact) {
+#ifdef BPSX_PHASE_TIMING
+      for (int k = 0; k < 8; ++k) g.phase[k] = 0;
+      g.phase_t0 = __builtin_readcyclecounter();
+#endif
       st.ol.init();
-      st.ol.template update<false>(startIp << 11, __float_as_uint(total));
+      st.ol.template update<false>(startIp << 11, __float_as_uint(total), lane);
       st.ol.template count<false>();
       st.logEnd = st.synced = 0;
       // the loop is instantiated for links in LDS only or spilling, and for a list within one
@@ -1345,6 +1375,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         st.ol.n0 = wlane(st.ol.n0, front, p);
         resolved = true;
       }
+#ifdef BPSX_PHASE_TIMING
+      for (int k = 0; k < 8; ++k) phase_acc[k] += g.phase[k];
+      phase_t0 = __builtin_readcyclecounter();
+#endif
       if (restart) {
         // the heap outgrew the registers during the replay: the search runs again with the exact loops
         g.exactRuns++;

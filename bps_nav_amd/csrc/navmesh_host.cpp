@@ -155,11 +155,11 @@ int parse_navmesh(const uint8_t* b, size_t n, HostScene* out) {
     }
   }
   // per-edge records of the path search
-  s.aedges.assign((size_t)np * kNvp, AEdge{{0, 0, 0}, kNoNb});
+  s.aedges.assign((size_t)np * kEdgeStride, AEdge{{0, 0, 0}, kNoNb});
   for (int i = 0; i < np; ++i) {
     const PolyRec& r = s.polys[i];
     for (int k = 0; k < r.nv; ++k) {
-      AEdge& e = s.aedges[(size_t)i * kNvp + k];
+      AEdge& e = s.aedges[(size_t)i * kEdgeStride + k];
       const float* l = r.v[k];
       const float* rt = r.v[(k + 1) % r.nv];
       for (int c = 0; c < 3; ++c) e.mid[c] = (l[c] + rt[c]) * 0.5f;

@@ -11,7 +11,7 @@ namespace bpsx {
 
 struct HostScene {
   std::vector<PolyRec> polys;     // tri_base / dvert_base are scene-relative until upload
-  std::vector<AEdge> aedges;      // [polygon][kNvp]
+  std::vector<AEdge> aedges;      // [polygon][kEdgeStride]
   std::vector<BVNodeDev> bv;
   std::vector<uint8_t> dtris;     // [.][4]
   std::vector<float> dverts;      // [.][3]
