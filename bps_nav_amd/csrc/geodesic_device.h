@@ -1062,7 +1062,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
 #ifdef BPSX_BRIDGE_AT
     if (ol.size > BPSX_BRIDGE_AT) return kAstarGrowHeap;   // test build: leave the sorted list early
 #endif
-    if (ol.size > (W ? 128 : 64) - kRows * kNvp) return kAstarGrowHeap;
     if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
     FM(0);
     // ---- how many entries at the front are each the only one with their total
@@ -1187,6 +1186,9 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     tb = rowIn ? tb : 0xffffffffu;
     const bool update = tb != 0xffffffffu;
     const bool isNew = update && ni < 0;   // a new node is always taken
+    unsigned long long upd = lanes_where(tb != 0xffffffffu);
+    // nothing has changed yet: a list that would outgrow its registers goes on in the wider instantiation
+    if (__builtin_expect(ol.size - c + __popcll(upd) > (W ? 128 : 64), 0)) return kAstarGrowHeap;
     (*pops) += (uint32_t)c;
     // the committed rows' nodes are closed
     if (el == 0 && rowIn) g.set_link<S>(bi, with_flags(blink, 2u));
@@ -1246,7 +1248,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     // ---- the open list: the committed entries leave, the updates enter
     ol.template drop_front<W>(c, lane);
     const uint32_t packed = (uint32_t)ni | (nb << 11);
-    unsigned long long upd = lanes_where(tb != 0xffffffffu);
     {
       // the pass in the operation log: the header from an idle lane, the updates in lane order
       const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(upd >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)upd, 0u));

@@ -485,6 +485,7 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
 #ifdef BPSX_QUERY_TRACE
   const unsigned long long trace_t0 = wall_clock64();
   g.missTop = g.missNb = g.maxHeap = 0;
+  const uint32_t trace_replays0 = g.tieReplays, trace_spills0 = g.linkSpills, trace_bridges0 = g.heapSpills + g.exactRuns;
   const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
   // the longer the expected search, the sooner its instructions issue; a search of unknown
@@ -500,8 +501,9 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
     const unsigned int ti = atomicAdd(&g_trace_n, 1u);
     if (ti < (1u << 17)) {
       g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = T.pops - pops0;
-      g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)(g.missTop & 0xfffu) << 24) |
-                        ((unsigned long long)(g.missNb & 0xfffu) << 36) | ((unsigned long long)(g.maxHeap & 0xffu) << 48);
+      // class, predicted length, ties resolved from the log, link spills, bridges to the exact loops
+      g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)((g.tieReplays - trace_replays0) & 0xfffu) << 24) |
+                        ((unsigned long long)((g.linkSpills - trace_spills0) & 0xfffu) << 36) | ((unsigned long long)((g.heapSpills + g.exactRuns - trace_bridges0) & 0xffu) << 48);
     }
 #endif
     out[q.out] = d;
