@@ -294,11 +294,13 @@ struct RegHeap {
 // of all lanes with the new total and a shift of those above it.  Unused places hold kEmpty
 // keys and kNone nodes.  Entries with equal totals sit next to each other in no defined order.
 struct OpenList {
-  uint32_t t0, n0, t1, n1;   // totals as bit patterns (see RegHeap), nodes packed like RegHeap's
+  static constexpr int kPairs = 4;
+  uint32_t t[kPairs], n[kPairs];   // totals as bit patterns (see RegHeap), nodes packed like RegHeap's
   int size;
   static constexpr uint32_t kEmpty = 0x7fffffffu;
   static constexpr uint32_t kNone = 0xffffffffu;    // no packed node looks like this (26 bits)
-  BPSX_DEV void init() { t0 = t1 = kEmpty; n0 = n1 = kNone; size = 0; }
+  BPSX_DEV void init() { t[0] = kEmpty; n[0] = kNone; size = 0; }   // further pairs are cleared when the list grows into them
+  BPSX_DEV void clear_pair(int k) { t[k] = kEmpty; n[k] = kNone; }
   // lane L takes v of lane L - 1, lane 0 keeps `first`
   static BPSX_DEV uint32_t up1(uint32_t first, uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp((int)first, (int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
@@ -313,53 +315,74 @@ struct OpenList {
     asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(mask));
     return r;
   }
-  // The first c entries leave (W false: the list lives in the first pair only).
-  template <bool W> BPSX_DEV void drop_front(int c, int lane) {
-    if (!W) {
-      for (int i = 0; i < c; ++i) { t0 = down1(kEmpty, t0); n0 = down1(kNone, n0); }
+  // The first c entries leave.  P: register pairs in use (64 entries each).
+  template <int P> BPSX_DEV void drop_front(int c, int lane) {
+    if (P == 1) {
+      for (int i = 0; i < c; ++i) { t[0] = down1(kEmpty, t[0]); n[0] = down1(kNone, n[0]); }
     } else {
       const int src = ((lane + c) & 63) * 4;
-      const uint32_t a0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)t0), b0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)n0);
-      const uint32_t a1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)t1), b1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)n1);
+      uint32_t a[P], b[P];
+#pragma unroll
+      for (int k = 0; k < P; ++k) { a[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)t[k]); b[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)n[k]); }
       const bool same = lane + c < 64;
-      t0 = same ? a0 : a1; n0 = same ? b0 : b1;
-      t1 = same ? a1 : kEmpty; n1 = same ? b1 : kNone;
+#pragma unroll
+      for (int k = 0; k < P; ++k) {
+        t[k] = same ? a[k] : (k + 1 < P ? a[k + 1 < P ? k + 1 : k] : kEmpty);
+        n[k] = same ? b[k] : (k + 1 < P ? b[k + 1 < P ? k + 1 : k] : kNone);
+      }
     }
   }
   // the number of entries, after drops and updates (which do not keep it)
-  template <bool W> BPSX_DEV void count() {
-    size = __popcll(lanes_where(t0 != kEmpty));
-    if (W) size += __popcll(lanes_where(t1 != kEmpty));
+  template <int P> BPSX_DEV void count() {
+    size = 0;
+#pragma unroll
+    for (int k = 0; k < P; ++k) size += __popcll(lanes_where(t[k] != kEmpty));
   }
   // lane L takes v of lane L - 1 (lane 0: anything)
   static BPSX_DEV uint32_t from_below(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, true);
   }
-  // Node n gets total t: its entry, if it has one, leaves, and the new entry goes behind those
-  // with totals up to t.  (A node has an entry exactly when it is open and has not just been
+  // Node n_ gets total t_: its entry, if it has one, leaves, and the new entry goes behind those
+  // with totals up to t_.  (A node has an entry exactly when it is open and has not just been
   // taken off the front, so whether this is the reference's push or its modify need not be told.)
-  // No branches: without an old entry the "entries up to the old place" are all entries.
-  template <bool W> BPSX_DEV void update(uint32_t n, uint32_t t, int lane) {
-    const unsigned long long g0 = lanes_where(t0 > t), h0 = lanes_where(n0 == n);
-    if (!W) {
-      // without an old entry its place is -1: as an unsigned bound that keeps every lane
+  template <int P> BPSX_DEV void update(uint32_t n_, uint32_t t_, int lane) {
+    if (P == 1) {
+      // No branches: without an old entry its place is -1, as an unsigned bound that keeps every lane
+      const unsigned long long g0 = lanes_where(t[0] > t_), h0 = lanes_where(n[0] == n_);
       const unsigned long long m0 = g0 & lanes_where((uint32_t)lane <= (uint32_t)first_lane(h0));
       const int p = first_lane(m0);   // never empty: the unused places compare greater
-      t0 = pick(m0, from_below(t0), t0);
-      n0 = pick(m0, from_below(n0), n0);
-      wlane2(t0, t, n0, n, p);
+      t[0] = pick(m0, from_below(t[0]), t[0]);
+      n[0] = pick(m0, from_below(n[0]), n[0]);
+      wlane2(t[0], t_, n[0], n_, p);
       return;
     }
-    const unsigned long long g1 = lanes_where(t1 > t), h1 = lanes_where(n1 == n);
-    unsigned long long m0 = g0, m1 = g1;
-    if (h0) { m0 &= (2ull << (__ffsll((long long)h0) - 1)) - 1ull; m1 = 0; }
-    else if (h1) m1 &= (2ull << (__ffsll((long long)h1) - 1)) - 1ull;
-    const int p = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
-    const uint32_t ct = rlane(t0, 63), cn = rlane(n0, 63);   // what moves up into the second pair
-    t1 = pick(m1, up1(ct, t1), t1); n1 = pick(m1, up1(cn, n1), n1);
-    t0 = pick(m0, from_below(t0), t0); n0 = pick(m0, from_below(n0), n0);
-    if (p < 64) { t0 = wlane(t0, t, p); n0 = wlane(n0, n, p); }
-    else { t1 = wlane(t1, t, p - 64); n1 = wlane(n1, n, p - 64); }
+    unsigned long long m[P];
+    int rp = -1, rl = 0;   // pair and lane of the old entry
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+      m[k] = lanes_where(t[k] > t_);
+      const unsigned long long h = lanes_where(n[k] == n_);
+      if (h && rp < 0) { rp = k; rl = __ffsll((long long)h) - 1; }
+    }
+    // only the entries from the new place up to the old one move
+    int pp = -1, pl = 0;   // pair and lane of the new place
+#pragma unroll
+    for (int k = 0; k < P; ++k) {
+      if (rp >= 0 && k > rp) m[k] = 0;
+      if (k == rp) m[k] &= (2ull << rl) - 1ull;
+      if (m[k] && pp < 0) { pp = k; pl = __ffsll((long long)m[k]) - 1; }
+    }
+#pragma unroll
+    for (int k = P - 1; k >= 1; --k) {
+      const uint32_t ct = rlane(t[k - 1], 63), cn = rlane(n[k - 1], 63);   // what moves up into pair k
+      t[k] = pick(m[k], up1(ct, t[k]), t[k]);
+      n[k] = pick(m[k], up1(cn, n[k]), n[k]);
+    }
+    t[0] = pick(m[0], from_below(t[0]), t[0]);
+    n[0] = pick(m[0], from_below(n[0]), n[0]);
+#pragma unroll
+    for (int k = 0; k < P; ++k)
+      if (pp == k) wlane2(t[k], t_, n[k], n_, pl);
   }
 };
 
@@ -1037,7 +1060,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
 // node of an earlier one (it sees it as open, the reference as closed): both views lead to
 // the same node state and the same list, because a modify that finds no entry is a push.
 // Returns kAstarTie when the first two entries share the smallest total.
-template <bool S, bool W>
+template <bool S, int P>
 BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops,
                              bool frontResolved) {
   const int lane = g.lane;
@@ -1065,9 +1088,9 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
     FM(0);
     // ---- how many entries at the front are each the only one with their total
-    const unsigned long long uniq = lanes_where(ol.t0 < OpenList::down1(OpenList::kEmpty, ol.t0));
+    const unsigned long long uniq = lanes_where(ol.t[0] < OpenList::down1(OpenList::kEmpty, ol.t[0]));
     int lim = __builtin_ctzll(~uniq | (1ull << kRows));
-    const uint32_t cand = (uint32_t)__builtin_amdgcn_ds_bpermute(row * 4, (int)ol.n0);   // entry `row`
+    const uint32_t cand = (uint32_t)__builtin_amdgcn_ds_bpermute(row * 4, (int)ol.n[0]);   // entry `row`
     const int bi = (int)(cand & 0x7ffu);
     const uint32_t ip = cand >> 11;
     const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
@@ -1160,7 +1183,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     int c = lim;
     bool pairFails = false;
     if (lim > 1) {
-      const uint32_t k1 = rlane(ol.t0, 1), k2 = rlane(ol.t0, 2), k3 = rlane(ol.t0, 3);
+      const uint32_t k1 = rlane(ol.t[0], 1), k2 = rlane(ol.t[0], 2), k3 = rlane(ol.t[0], 3);
       const unsigned long long v1 = lanes_where(tb <= k1) & rowsAt1;
       const unsigned long long v2 = lanes_where(tb <= k2) & kRows2;
       const unsigned long long v3 = lanes_where(tb <= k3) & kRows3;
@@ -1188,7 +1211,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const bool isNew = update && ni < 0;   // a new node is always taken
     unsigned long long upd = lanes_where(tb != 0xffffffffu);
     // nothing has changed yet: a list that would outgrow its registers goes on in the wider instantiation
-    if (__builtin_expect(ol.size - c + __popcll(upd) > (W ? 128 : 64), 0)) return kAstarGrowHeap;
+    if (__builtin_expect(ol.size - c + __popcll(upd) > 64 * P, 0)) return kAstarGrowHeap;
     (*pops) += (uint32_t)c;
     // the committed rows' nodes are closed
     if (el == 0 && rowIn) g.set_link<S>(bi, with_flags(blink, 2u));
@@ -1246,7 +1269,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     wave_sync();
     FM(8);
     // ---- the open list: the committed entries leave, the updates enter
-    ol.template drop_front<W>(c, lane);
+    ol.template drop_front<P>(c, lane);
     const uint32_t packed = (uint32_t)ni | (nb << 11);
     {
       // the pass in the operation log: the header from an idle lane, the updates in lane order
@@ -1266,9 +1289,9 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     while (upd) {
       const int src = first_lane(upd);
       upd = without_lane(upd, src);
-      ol.template update<W>(rlane(packed, src), rlane(tb, src), lane);
+      ol.template update<P>(rlane(packed, src), rlane(tb, src), lane);
     }
-    ol.template count<W>();
+    ol.template count<P>();
     FM(10);
   }
 }
@@ -1333,18 +1356,27 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       g.phase_t0 = __builtin_readcyclecounter();
 #endif
       st.ol.init();
-      st.ol.template update<false>(startIp << 11, __float_as_uint(total), lane);
-      st.ol.template count<false>();
+      st.ol.template update<1>(startIp << 11, __float_as_uint(total), lane);
+      st.ol.template count<1>();
       st.logEnd = st.synced = 0;
       // the loop is instantiated for links in LDS only or spilling, and for a list within one
       // register pair or two; a search moves on when one more pass could outgrow what it runs in
       bool resolved = false, restart = false;
+      int pairs = 1;   // register pairs of the list in use
       for (;;) {
-        if (!spill) ex = wide ? astar_fast<false, true>(g, st, edges, endIp, endPos, pops, resolved) : astar_fast<false, false>(g, st, edges, endIp, endPos, pops, resolved);
-        else ex = wide ? astar_fast<true, true>(g, st, edges, endIp, endPos, pops, resolved) : astar_fast<true, false>(g, st, edges, endIp, endPos, pops, resolved);
+#define BPSX_FAST_RUN(SP) (pairs == 1 ? astar_fast<SP, 1>(g, st, edges, endIp, endPos, pops, resolved) : \
+                           pairs == 2 ? astar_fast<SP, 2>(g, st, edges, endIp, endPos, pops, resolved) : \
+                                        astar_fast<SP, 4>(g, st, edges, endIp, endPos, pops, resolved))
+        ex = spill ? BPSX_FAST_RUN(true) : BPSX_FAST_RUN(false);
+#undef BPSX_FAST_RUN
         resolved = false;
         if (ex == kAstarGrowLinks) { g.linkSpills++; spill = true; continue; }
-        if (ex == kAstarGrowHeap && !wide) { wide = true; continue; }
+        if (ex == kAstarGrowHeap && pairs < OpenList::kPairs) {
+          // the list grows into further registers, empty so far
+          if (pairs == 1) { st.ol.clear_pair(1); pairs = 2; }
+          else { st.ol.clear_pair(2); st.ol.clear_pair(3); pairs = 4; }
+          continue;
+        }
         if (ex != kAstarTie && ex != kAstarGrowHeap && ex != kAstarLogFull) break;
         // the reference's heap is needed: bring it up to date from the log
         if (!replay_log(g.ws->oplog, st, lane) || st.rh.size != st.ol.size) { restart = true; break; }
@@ -1355,7 +1387,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
           int badKey = 0, badNode = 0;
           for (int i = 0; i < st.ol.size; ++i) {
             const uint32_t hk = rlane(copy.t0, 1), hn = rlane(copy.n0, 1);
-            const uint32_t lk = i < 64 ? rlane(st.ol.t0, i) : rlane(st.ol.t1, i - 64), ln = i < 64 ? rlane(st.ol.n0, i) : rlane(st.ol.n1, i - 64);
+            const uint32_t lk = i < 64 ? rlane(st.ol.t[0], i) : rlane(st.ol.t[1], i - 64), ln = i < 64 ? rlane(st.ol.n[0], i) : rlane(st.ol.n[1], i - 64);
             if (hk != lk) badKey++;
             else if (hn != ln) badNode++;
             copy.pop(lane);
@@ -1368,12 +1400,12 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         // a tie: the reference pops what its heap has at the root.  That entry goes first.
         g.tieReplays++;
         const uint32_t root = rlane(st.rh.n0, 1);
-        const unsigned long long at = lanes_where(st.ol.n0 == root);
+        const unsigned long long at = lanes_where(st.ol.n[0] == root);
         const int p = at ? __ffsll((long long)at) - 1 : -1;
-        if (p < 0 || rlane(st.ol.t0, p) != rlane(st.ol.t0, 0)) { restart = true; break; }
-        const uint32_t front = rlane(st.ol.n0, 0);
-        st.ol.n0 = wlane(st.ol.n0, root, 0);
-        st.ol.n0 = wlane(st.ol.n0, front, p);
+        if (p < 0 || rlane(st.ol.t[0], p) != rlane(st.ol.t[0], 0)) { restart = true; break; }
+        const uint32_t front = rlane(st.ol.n[0], 0);
+        st.ol.n[0] = wlane(st.ol.n[0], root, 0);
+        st.ol.n[0] = wlane(st.ol.n[0], front, p);
         resolved = true;
       }
 #ifdef BPSX_PHASE_TIMING
