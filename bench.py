@@ -248,7 +248,7 @@ def main():
     K = P   # the counters below cover the profiled pass
     log(f"per step: {d['geodesic_queries'] / K:.0f} geodesic queries, {d['astar_pops'] / max(1, d['geodesic_queries']):.0f} "
         f"A* pops/query, corridor {d['corridor_polys'] / max(1, d['geodesic_queries']):.1f} polys/query, "
-        f"{d['resets'] / K:.1f} resets, {d.get('geo_link_spills', 0) / K:.0f} link spills, {d.get('geo_heap_spills', 0) / K:.0f} heap spills, {d.get('geo_long_path', 0) / K:.0f} on the large-LDS path, {d.get('geo_exact_runs', 0) / K:.0f} run again with the exact heap, {d.get('geo_tie_replays', 0) / K:.0f} ties resolved from the log; non-finite distances now: {int((~np.isfinite(dist)).sum())} of {N}")
+        f"{d['resets'] / K:.1f} resets, {d.get('geo_link_spills', 0) / K:.0f} link spills, {d.get('geo_heap_spills', 0) / K:.0f} heap spills, {d.get('geo_long_path', 0) / K:.0f} on the large-LDS path, {d.get('geo_exact_runs', 0) / K:.0f} run again with the exact heap, {d.get('geo_pair_ties', 0) / K:.0f} tied pairs taken in one pass, {d.get('geo_tie_replays', 0) / K:.0f} ties resolved from the log; non-finite distances now: {int((~np.isfinite(dist)).sum())} of {N}")
     # roofline of the dominant kernel (geodesic over the step's queries), HIP-event timed
     dominant = max(kt, key=kt.get)
     geo_bytes = BYTES_PER_CORRIDOR_POLY * d["corridor_polys"] + BYTES_PER_QUERY_ENDS * d["geodesic_queries"]

@@ -250,14 +250,14 @@ class PointNavRolloutGenerator:
         _lib.check(self._L.bpsx_check_errors(self._h))
 
     def counters(self):
-        out = np.zeros(21, np.uint64)
+        out = np.zeros(22, np.uint64)
         _lib.check(self._L.bpsx_get_counters(self._h, out.ctypes.data))
         names = ["agent_steps", "forward_moves", "geodesic_queries", "astar_pops", "corridor_polys", "resets",
                  "move_polys", "snap_candidates"]
         d = dict(zip(names, (int(v) for v in out[:8])))
         d["phase_cycles"] = [int(v) for v in out[8:16]]
         d["geo_link_spills"], d["geo_heap_spills"], d["geo_long_path"] = int(out[16]), int(out[17]), int(out[18])
-        d["geo_exact_runs"], d["geo_tie_replays"] = int(out[19]), int(out[20])
+        d["geo_exact_runs"], d["geo_tie_replays"], d["geo_pair_ties"] = (int(v) for v in out[19:22])
         return d
 
     def set_profiling(self, enabled):

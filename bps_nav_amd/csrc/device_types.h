@@ -192,7 +192,7 @@ constexpr uint32_t kCostUnknown = 0xffffffffu;
 
 enum Counter {
   kCntSteps = 0, kCntForward, kCntGeoQueries, kCntAstarPops, kCntCorridor, kCntResets, kCntMovePolys, kCntSnapCands,
-  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18, kCntExactRuns = 19, kCntTieReplays = 20   // 8..15: phase cycles of the diagnostic build
+  kCntLinkSpills = 16, kCntHeapSpills = 17, kCntLongPath = 18, kCntExactRuns = 19, kCntTieReplays = 20, kCntPairTies = 21   // 8..15: phase cycles of the diagnostic build
 };
 
 }  // namespace bpsx

@@ -524,6 +524,7 @@ struct GeoWave {
 #endif
   uint32_t exactRuns;                // queries run again with the exact heap
   uint32_t tieReplays;               // ties resolved by replaying the operation log through the exact heap
+  uint32_t pairTies;                 // passes that took two nodes of equal total in one go
 #ifdef BPSX_QUERY_TRACE
   uint32_t missTop, missNb, maxHeap;
 #endif
@@ -1082,9 +1083,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
   for (;;) {
     if (ol.size <= 0) return kAstarEmpty;
     if (!S && g.nodeCount > kLinksLds - kRows * kNvp) return kAstarGrowLinks;
-#ifdef BPSX_BRIDGE_AT
-    if (ol.size > BPSX_BRIDGE_AT) return kAstarGrowHeap;   // test build: leave the sorted list early
-#endif
     if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
     FM(0);
     // ---- how many entries at the front are each the only one with their total
@@ -1106,6 +1104,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         // way: the pass takes both and notes in the log that their order is open.
         if (!(uniq & 2ull)) return kAstarTie;
         pairTie = true;
+        g.pairTies++;   // counts the attempts: one that fails comes back through the log
         rowsAt1 = kRows2;
         lim = __builtin_ctzll(~(uniq | 3ull) | (1ull << kRows));
       }
@@ -1377,27 +1376,13 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
           else { st.ol.clear_pair(2); st.ol.clear_pair(3); pairs = 4; }
           continue;
         }
-        if (ex != kAstarTie && ex != kAstarGrowHeap && ex != kAstarLogFull) break;
-        // the reference's heap is needed: bring it up to date from the log
+        // a list beyond the registers or a full log (neither met in the benchmark configurations'
+        // mazes and rooms, both in a hall without obstacles): the search runs again with the exact loops
+        if (ex == kAstarGrowHeap || ex == kAstarLogFull) { restart = true; break; }
+        if (ex != kAstarTie) break;
+        // a tie: the reference pops what its heap has at the root, so the heap is brought up to
+        // date from the log, and that entry goes first
         if (!replay_log(g.ws->oplog, st, lane) || st.rh.size != st.ol.size) { restart = true; break; }
-#ifdef BPSX_VERIFY_REPLAY
-        {
-          // popping a copy of the rebuilt heap must give the list's entries in order
-          RegHeap copy = st.rh;
-          int badKey = 0, badNode = 0;
-          for (int i = 0; i < st.ol.size; ++i) {
-            const uint32_t hk = rlane(copy.t0, 1), hn = rlane(copy.n0, 1);
-            const uint32_t lk = i < 64 ? rlane(st.ol.t[0], i) : rlane(st.ol.t[1], i - 64), ln = i < 64 ? rlane(st.ol.n[0], i) : rlane(st.ol.n[1], i - 64);
-            if (hk != lk) badKey++;
-            else if (hn != ln) badNode++;
-            copy.pop(lane);
-          }
-          if (badKey) g.exactRuns += 1000000;
-          if (badNode) g.exactRuns += 1000;
-        }
-#endif
-        if (ex != kAstarTie) { g.heapSpills++; break; }   // the list or the log is full: on with the exact loops
-        // a tie: the reference pops what its heap has at the root.  That entry goes first.
         g.tieReplays++;
         const uint32_t root = rlane(st.rh.n0, 1);
         const unsigned long long at = lanes_where(st.ol.n[0] == root);
@@ -1413,14 +1398,12 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       phase_t0 = __builtin_readcyclecounter();
 #endif
       if (restart) {
-        // the heap outgrew the registers during the replay: the search runs again with the exact loops
         g.exactRuns++;
         *pops = pops0;
         exact = true;
         continue;
       }
-      if (ex != kAstarGrowHeap && ex != kAstarLogFull) break;
-      // st.rh is the reference's heap as of now: the exact loops carry on from here
+      break;
     }
 #ifdef BPSX_ONE_NODE_PER_PASS
     ex = ASTAR_RUN(0);
@@ -1458,9 +1441,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
 #undef ASTAR_ARGS
   // an open list that ran empty, or a pool that ran out, is DT_PARTIAL_RESULT or
   // DT_OUT_OF_NODES in the reference: no path to build, the result is a failure
-#ifdef BPSX_DEBUG_BRIDGE
-  if (ex != kAstarGoal || st.outOfNodes) return -(1 + (int)ex + 10 * (int)st.outOfNodes + 100 * st.rh.size + 100000 * (int)(*pops - pops0));
-#endif
   if (ex != kAstarGoal || st.outOfNodes) return 0;
   const int lastBest = st.lastBest;
   // getPathToNode: one walk up the parents notes the node indices (in the window's array of
@@ -1606,9 +1586,6 @@ BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q,
   unsigned long long phase_t0 = __builtin_readcyclecounter();
 #else
   const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops);
-#endif
-#ifdef BPSX_DEBUG_BRIDGE
-  if (n < 0) return (float)n;
 #endif
   if (n <= 0) return INF;
   *corridor += (uint32_t)n;

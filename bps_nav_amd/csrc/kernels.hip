@@ -485,7 +485,7 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
 #ifdef BPSX_QUERY_TRACE
   const unsigned long long trace_t0 = wall_clock64();
   g.missTop = g.missNb = g.maxHeap = 0;
-  const uint32_t trace_replays0 = g.tieReplays, trace_spills0 = g.linkSpills, trace_bridges0 = g.heapSpills + g.exactRuns;
+  const uint32_t trace_replays0 = g.tieReplays, trace_spills0 = g.linkSpills, trace_bridges0 = g.exactRuns;
   const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
   // the longer the expected search, the sooner its instructions issue; a search of unknown
@@ -503,7 +503,7 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
       g_trace[ti][0] = trace_t0; g_trace[ti][1] = wall_clock64(); g_trace[ti][2] = T.pops - pops0;
       // class, predicted length, ties resolved from the log, link spills, bridges to the exact loops
       g_trace[ti][3] = (unsigned long long)cls | ((trace_pred & 0xffffu) << 8) | ((unsigned long long)((g.tieReplays - trace_replays0) & 0xfffu) << 24) |
-                        ((unsigned long long)((g.linkSpills - trace_spills0) & 0xfffu) << 36) | ((unsigned long long)((g.heapSpills + g.exactRuns - trace_bridges0) & 0xffu) << 48);
+                        ((unsigned long long)((g.linkSpills - trace_spills0) & 0xfffu) << 36) | ((unsigned long long)((g.exactRuns - trace_bridges0) & 0xffu) << 48);
     }
 #endif
     out[q.out] = d;
@@ -540,7 +540,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   for (int c = 0; c < kGeoClasses; ++c) first[c + 1] = first[c] + (uint32_t)uniform_i((int)counts[c]);
   const uint32_t nq = first[kGeoClasses], nlong = first[kLongClasses];
   GeoTotals T;
-  uint32_t linkSpills = 0, heapSpills = 0, exactRuns = 0, tieReplays = 0;
+  uint32_t linkSpills = 0, heapSpills = 0, exactRuns = 0, tieReplays = 0, pairTies = 0;
   if (threadIdx.x == 0) long_ticket = atomicAdd(head_long, 1u);
   __syncthreads();
   const uint32_t lt = (uint32_t)uniform_i((int)long_ticket);
@@ -552,12 +552,12 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     gl.ws = slot;
     gl.heapSize = 0;
     gl.nodeCount = 0;
-    gl.linkSpills = gl.heapSpills = gl.exactRuns = gl.tieReplays = 0;
+    gl.linkSpills = gl.heapSpills = gl.exactRuns = gl.tieReplays = gl.pairTies = 0;
     int cls = 0;
     while (lt >= first[cls + 1]) cls++;
     const GeoQuery q = queries[(size_t)cls * stride + (lt - first[cls])];
     serve_query(gl, nav, q, cls, out, last_cost, T);
-    linkSpills += gl.linkSpills; heapSpills += gl.heapSpills; exactRuns += gl.exactRuns; tieReplays += gl.tieReplays;
+    linkSpills += gl.linkSpills; heapSpills += gl.heapSpills; exactRuns += gl.exactRuns; tieReplays += gl.tieReplays; pairTies += gl.pairTies;
     if (lane == 0) atomicAdd((unsigned long long*)&counters[kCntLongPath], 1ull);
   }
   geo::GeoWave g;
@@ -566,7 +566,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   g.ws = slot;
   g.heapSize = 0;
   g.nodeCount = 0;
-  g.linkSpills = g.heapSpills = g.exactRuns = g.tieReplays = 0;
+  g.linkSpills = g.heapSpills = g.exactRuns = g.tieReplays = g.pairTies = 0;
   // tickets below `taken` went to the blocks' first wavefronts above
   const uint32_t taken = nlong < gridDim.x ? nlong : gridDim.x;
   for (;;) {
@@ -580,7 +580,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     const GeoQuery q = queries[(size_t)cls * stride + (qi - first[cls])];
     serve_query(g, nav, q, cls, out, last_cost, T);
   }
-  linkSpills += g.linkSpills; heapSpills += g.heapSpills; exactRuns += g.exactRuns; tieReplays += g.tieReplays;
+  linkSpills += g.linkSpills; heapSpills += g.heapSpills; exactRuns += g.exactRuns; tieReplays += g.tieReplays; pairTies += g.pairTies;
   if (lane == 0 && T.done) {
     atomicAdd((unsigned long long*)&counters[kCntGeoQueries], (unsigned long long)T.done);
     atomicAdd((unsigned long long*)&counters[kCntAstarPops], (unsigned long long)T.pops);
@@ -589,6 +589,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     if (heapSpills) atomicAdd((unsigned long long*)&counters[kCntHeapSpills], (unsigned long long)heapSpills);
     if (exactRuns) atomicAdd((unsigned long long*)&counters[kCntExactRuns], (unsigned long long)exactRuns);
     if (tieReplays) atomicAdd((unsigned long long*)&counters[kCntTieReplays], (unsigned long long)tieReplays);
+    if (pairTies) atomicAdd((unsigned long long*)&counters[kCntPairTies], (unsigned long long)pairTies);
 #ifdef BPSX_PHASE_TIMING
     for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], T.phase_acc[k]);
 #endif

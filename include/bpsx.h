@@ -175,11 +175,15 @@ int bpsx_check_errors(bpsx_sim *sim);
  * more node links than the kernel keeps in LDS, [17] path searches whose open list outgrew
  * the kernel's registers (both continue in slower code; results are the same), [18] path
  * searches expected to be among the longest of their step, which the kernel runs with larger
- * LDS structures (same results), [19] path searches run a second time with the reference's
- * open-list arrangement throughout, [20] times two open nodes shared the smallest total and
- * the reference's arrangement was rebuilt from the search's operation log to tell which comes
- * first (same results either way). */
-#define BPSX_NUM_COUNTERS 21
+ * LDS structures (same results).  The path search keeps its open list sorted by total instead of
+ * in the reference's heap arrangement, which only matters when two open nodes share the
+ * smallest total: [21] counts the passes that found such a pair and tried to expand both at once
+ * (possible when neither affects the other), [20] the times the reference's arrangement had to be
+ * rebuilt from the search's operation log to tell which of the two comes first, [19] the searches
+ * run a second time with the reference's heap throughout, because the open list outgrew the
+ * sorted form's 256 entries or the heap outgrew the registers during a rebuild.  Same results in
+ * all cases. */
+#define BPSX_NUM_COUNTERS 22
 int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
 /* Per-kernel timing with HIP events on the step's own stream. While enabled, every
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
