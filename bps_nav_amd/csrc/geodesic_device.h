@@ -1200,7 +1200,24 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const uint32_t jc = (uint32_t)first_lane(lanes_where(seenr < (uint32_t)row)) >> 4;   // none: far above 4
       c = jc < (uint32_t)c ? (int)jc : c;
       // rows 0 and 1 of a tied pair in either order: row 0 must not read what row 1 updates either
-      if (__builtin_expect(pairTie, 0)) pairFails = c < 2 || (lanes_where(seenr == 1u) & kRows1) != 0;
+      if (__builtin_expect(pairTie, 0)) {
+        pairFails = c < 2 || (lanes_where(seenr == 1u) & kRows1) != 0;
+        if (pairFails && jv >= 2) {
+          // The marks are kept per polygon hash, and a pair that fails costs a replay of the log:
+          // the polygons that either row updates are compared with those the other row reads,
+          // and a clash that was two polygons with one hash lets the pair (and only it) stand.
+          const uint32_t readPoly = ownLane ? (rowOn ? ip : 0xffffffffu) : (valid ? nb : 0xffffffffu);
+          unsigned long long w = lanes_where(tb != 0xffffffffu) & kRows2;
+          bool real = false;
+          while (w) {
+            const int src = first_lane(w);
+            w = without_lane(w, src);
+            const unsigned long long others = src < 16 ? (kRows2 & ~kRows1) : kRows1;
+            if (lanes_where(readPoly == rlane(nb, src)) & others) real = true;
+          }
+          if (!real) { pairFails = false; c = 2; }
+        }
+      }
     }
     if (__builtin_expect(pairFails, 0)) return kAstarTie;
     FM(5);
