@@ -525,6 +525,12 @@ struct GeoWave {
   uint32_t exactRuns;                // queries run again with the exact heap
   uint32_t tieReplays;               // ties resolved by replaying the operation log through the exact heap
   uint32_t pairTies;                 // passes that took two nodes of equal total in one go
+#ifdef BPSX_TIE_REASONS
+  uint32_t why[8];
+#define TIE_WHY(k) g.why[k]++
+#else
+#define TIE_WHY(k) do { } while (0)
+#endif
 #ifdef BPSX_QUERY_TRACE
   uint32_t missTop, missNb, maxHeap;
 #endif
@@ -1102,7 +1108,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         // whatever they put on the list lies above their total), the reference expands them one
         // after the other, in the order its heap has them in, and ends in the same state either
         // way: the pass takes both and notes in the log that their order is open.
-        if (!(uniq & 2ull)) return kAstarTie;
+        if (!(uniq & 2ull)) { TIE_WHY(0); return kAstarTie; }
         pairTie = true;
         g.pairTies++;   // counts the attempts: one that fails comes back through the log
         rowsAt1 = kRows2;
@@ -1115,7 +1121,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         return kAstarGoal;
       }
       if (goal) { const int jg = __builtin_ctzll(goal) >> 4; lim = jg < lim ? jg : lim; }
-      if (pairTie && lim < 2) return kAstarTie;   // the goal is one of the two
+      if (pairTie && lim < 2) { TIE_WHY(1); return kAstarTie; }   // the goal is one of the two
     }
     FM(1);
     const bool rowOn = row < lim;
@@ -1202,6 +1208,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       // rows 0 and 1 of a tied pair in either order: row 0 must not read what row 1 updates either
       if (__builtin_expect(pairTie, 0)) {
         pairFails = c < 2 || (lanes_where(seenr == 1u) & kRows1) != 0;
+        if (pairFails && jv < 2) TIE_WHY(2);
         if (pairFails && jv >= 2) {
           // The marks are kept per polygon hash, and a pair that fails costs a replay of the log:
           // the polygons that either row updates are compared with those the other row reads,
@@ -1215,7 +1222,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
             const unsigned long long others = src < 16 ? (kRows2 & ~kRows1) : kRows1;
             if (lanes_where(readPoly == rlane(nb, src)) & others) real = true;
           }
-          if (!real) { pairFails = false; c = 2; }
+          if (!real) { pairFails = false; c = 2; TIE_WHY(4); } else TIE_WHY(3);
         }
       }
     }

@@ -553,6 +553,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     gl.heapSize = 0;
     gl.nodeCount = 0;
     gl.linkSpills = gl.heapSpills = gl.exactRuns = gl.tieReplays = gl.pairTies = 0;
+#ifdef BPSX_TIE_REASONS
+    for (int k = 0; k < 8; ++k) gl.why[k] = 0;
+#endif
     int cls = 0;
     while (lt >= first[cls + 1]) cls++;
     const GeoQuery q = queries[(size_t)cls * stride + (lt - first[cls])];
@@ -567,6 +570,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   g.heapSize = 0;
   g.nodeCount = 0;
   g.linkSpills = g.heapSpills = g.exactRuns = g.tieReplays = g.pairTies = 0;
+#ifdef BPSX_TIE_REASONS
+  for (int k = 0; k < 8; ++k) g.why[k] = 0;
+#endif
   // tickets below `taken` went to the blocks' first wavefronts above
   const uint32_t taken = nlong < gridDim.x ? nlong : gridDim.x;
   for (;;) {
@@ -590,6 +596,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     if (exactRuns) atomicAdd((unsigned long long*)&counters[kCntExactRuns], (unsigned long long)exactRuns);
     if (tieReplays) atomicAdd((unsigned long long*)&counters[kCntTieReplays], (unsigned long long)tieReplays);
     if (pairTies) atomicAdd((unsigned long long*)&counters[kCntPairTies], (unsigned long long)pairTies);
+#ifdef BPSX_TIE_REASONS
+    for (int k = 0; k < 8; ++k) if (g.why[k]) atomicAdd((unsigned long long*)&counters[8 + k], (unsigned long long)g.why[k]);
+#endif
 #ifdef BPSX_PHASE_TIMING
     for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], T.phase_acc[k]);
 #endif
