@@ -1082,7 +1082,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
   constexpr unsigned long long kRowStart = 0x0001000100010001ull;
   constexpr unsigned long long kRows1 = 0xffffull, kRows2 = 0xffffffffull, kRows3 = 0xffffffffffffull;   // lanes of the first rows
   unsigned long long resolved = frontResolved ? 1ull : 0ull;
-  uint32_t warm = 0;   // see the prefetch below
   // Written for few instructions on the common path: what is rare sits behind one branch each,
   // and conditions that feed a ballot are folded into the compared value first, so that the
   // ballot is the comparison's own result.
@@ -1132,7 +1131,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const AEdge e = edges[ip * kEdgeStride + (uint32_t)el];
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
-    asm volatile("" ::"v"(warm));   // the previous pass's prefetch has a consumer: here, where the pass waits for memory anyway
     const int bis = rowOn ? bi : 0;
     const uint32_t blink = g.link<S>(bis);
     float b0, b1, b2, bcost;
@@ -1238,10 +1236,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     (*pops) += (uint32_t)c;
     // the committed rows' nodes are closed
     if (el == 0 && rowIn) g.set_link<S>(bi, with_flags(blink, 2u));
-    // The edge records of a polygon that enters the open list are asked for now: the scenes'
-    // records are far larger than the caches, and a node is expanded one pass later at the
-    // earliest, by which time its line (one per polygon) has arrived in L2.
-    if (update) warm = edges[nb * kEdgeStride].nb;
     FM(6);
     // ---- new nodes take consecutive indices in row and edge order
     {
