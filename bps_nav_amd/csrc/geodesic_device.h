@@ -1504,13 +1504,16 @@ BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const S
   float cs[3], ce[3];
   closest_on_poly_boundary(nav.polys[s.poly_base + F->corridor[0]], startPos, cs);
   closest_on_poly_boundary(nav.polys[s.poly_base + F->corridor[n - 1]], endPos, ce);
-  // straight-path points are only needed pairwise: keep the last one and the running length
+  // straight-path points are only needed pairwise: keep the last one and the running length.
+  // Every lane computes the same values; the conditions are taken through a ballot so that the
+  // control flow is the scalar unit's (no lane masks, no copies at the joins).
+  auto all = [](bool b) { return lanes_where(b) != 0; };
   float last[3] = {cs[0], cs[1], cs[2]};
   int npts = 1;
   float length = 0.0f;
   bool finished = false, overflow = false;
   auto append = [&](const float* p, bool isEnd) {
-    if (vequal(last, p)) return;  // merged with the previous point
+    if (all(vequal(last, p))) return;  // merged with the previous point
     const float dx = last[0] - p[0], dy = last[1] - p[1], dz = last[2] - p[2];
     length += sqrtf(dx * dx + (dy * dy + dz * dz));
     last[0] = p[0]; last[1] = p[1]; last[2] = p[2];
@@ -1530,13 +1533,13 @@ BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const S
         right[0] = p[3]; right[1] = p[4]; right[2] = p[5];
         if (i == 0) {
           float t;
-          if (dist_pt_seg_sqr2d(apex[0], apex[2], left, right, t) < 0.001f * 0.001f) continue;
+          if (all(dist_pt_seg_sqr2d(apex[0], apex[2], left, right, t) < 0.001f * 0.001f)) continue;
         }
       } else {
         left[0] = right[0] = ce[0]; left[1] = right[1] = ce[1]; left[2] = right[2] = ce[2];
       }
-      if (tri_area2d(apex, pr, right) <= 0.0f) {
-        if (vequal(apex, pr) || tri_area2d(apex, pl, right) > 0.0f) {
+      if (all(tri_area2d(apex, pr, right) <= 0.0f)) {
+        if (all(vequal(apex, pr)) || all(tri_area2d(apex, pl, right) > 0.0f)) {
           pr[0] = right[0]; pr[1] = right[1]; pr[2] = right[2];
           rightIsEnd = !(i + 1 < n);
           rightIndex = i;
@@ -1551,8 +1554,8 @@ BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const S
           continue;
         }
       }
-      if (tri_area2d(apex, pl, left) >= 0.0f) {
-        if (vequal(apex, pl) || tri_area2d(apex, pr, left) < 0.0f) {
+      if (all(tri_area2d(apex, pl, left) >= 0.0f)) {
+        if (all(vequal(apex, pl)) || all(tri_area2d(apex, pr, left) < 0.0f)) {
           pl[0] = left[0]; pl[1] = left[1]; pl[2] = left[2];
           leftIsEnd = !(i + 1 < n);
           leftIndex = i;
