@@ -159,6 +159,7 @@ struct alignas(128) GeoSlot {
   ANode nodes[kMaxNodes];
   HeapEntry heap_spill[kMaxNodes];
   OpRec oplog[kOpLogCap];
+  uint16_t parents[kMaxNodes];   // the nodes' parent indices once more, side by side: what the final walk up the path reads
 };
 
 struct GeoQuery {

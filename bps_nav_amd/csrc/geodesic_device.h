@@ -819,6 +819,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       }
       *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
       *reinterpret_cast<uint2*>(&hn.total) = make_uint2(__float_as_uint(total), (uint32_t)(bi + 1));   // total, parent = expanded node
+      g.ws->parents[ni] = (uint16_t)(bi + 1);
     }
     wave_sync();
     PHASE_MARK(5);
@@ -1017,6 +1018,7 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       }
       *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
       *reinterpret_cast<uint2*>(&hn.total) = make_uint2(__float_as_uint(total), parent);
+      g.ws->parents[ni] = (uint16_t)parent;
     }
     wave_sync();
     PHASE_MARK(5);
@@ -1282,6 +1284,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       }
       *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
       *reinterpret_cast<uint2*>(&hn.total) = make_uint2(tb, parent);
+      g.ws->parents[ni] = (uint16_t)parent;
     }
     wave_sync();
     FM(8);
@@ -1357,6 +1360,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       L->w_cost[0] = 0; L->w_total[0] = total;
       hn.cost = 0; hn.total = total;
       hn.parent = 0;
+      g.ws->parents[0] = 0;
       L->w_parent[0] = 0;
       L->n_link[0] = make_link(startIp, 1u, kChainEnd);   // open
       L->first[GeoWave::hash(startIp)] = 0;
@@ -1461,16 +1465,30 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
   // DT_OUT_OF_NODES in the reference: no path to build, the result is a failure
   if (ex != kAstarGoal || st.outOfNodes) return 0;
   const int lastBest = st.lastBest;
-  // getPathToNode: one walk up the parents notes the node indices (in the window's array of
-  // positions, no longer needed), then all lanes fill the corridor, which overlays the hash heads;
-  // the links stay readable while it is written
-  static_assert(sizeof(g.L->w_pos) >= kMaxPath * sizeof(uint16_t), "the walk must fit the array it reuses");
-  uint16_t* walk = reinterpret_cast<uint16_t*>(g.L->w_pos);
+  // getPathToNode: a walk up the parents notes the node indices, then all lanes fill the corridor,
+  // which overlays the hash heads; the links stay readable while it is written.  The walk is a
+  // chain of dependent reads, 70 of them on average: the parent indices, which HBM also holds
+  // side by side, are first copied into the window's arrays (no longer needed), so that the
+  // chain runs in LDS; a node beyond what fits there is read from HBM.
+  static_assert(offsetof(GeoLds, w_cost) == offsetof(GeoLds, w_total) + sizeof(GeoLds::w_total) &&
+                offsetof(GeoLds, w_pos) == offsetof(GeoLds, w_cost) + sizeof(GeoLds::w_cost), "the window's arrays must be contiguous");
+  constexpr int kParentsLds = (int)((sizeof(GeoLds::w_total) + sizeof(GeoLds::w_cost) + sizeof(GeoLds::w_pos)) / sizeof(uint16_t));
+  static_assert(sizeof(GeoLds::tag) >= kMaxPath * sizeof(uint16_t), "the walk must fit the array it reuses");
+  uint16_t* lparent = reinterpret_cast<uint16_t*>(g.L->w_total);
+  uint16_t* walk = reinterpret_cast<uint16_t*>(g.L->tag);
+  wave_sync();
+  const int inLds = g.nodeCount < kParentsLds ? g.nodeCount : kParentsLds;
+  {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(g.ws->parents);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(lparent);
+    for (int i = lane; i < (inLds + 1) / 2; i += 64) dst[i] = src[i];
+  }
   wave_sync();
   int length = 0;
-  for (int c = lastBest + 1; c && length <= kMaxNodes; c = uniform_i((int)g.ws->nodes[c - 1].parent)) {
+  for (int c = lastBest + 1; c && length <= kMaxNodes;) {
     if (lane == 0 && length < kMaxPath) walk[length] = (uint16_t)(c - 1);
     length++;
+    c = c - 1 < inLds ? uniform_i((int)lparent[c - 1]) : uniform_i((int)g.ws->parents[c - 1]);
   }
   wave_sync();
   const bool ok = length <= kMaxPath && link_id(g.link<true>(lastBest)) == endIp && !st.outOfNodes;
