@@ -1404,8 +1404,14 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         if (ex != kAstarTie) break;
         // a tie: the reference pops what its heap has at the root, so the heap is brought up to
         // date from the log, and that entry goes first
+#ifdef BPSX_TIE_REASONS
+        g.why[6] += (uint32_t)(st.logEnd - st.synced);   // records that the replay goes through
+#endif
         if (!replay_log(g.ws->oplog, st, lane) || st.rh.size != st.ol.size) { restart = true; break; }
         g.tieReplays++;
+#ifdef BPSX_TIE_REASONS
+        g.why[5] += *pops - pops0;   // nodes expanded so far when the log is replayed
+#endif
         const uint32_t root = rlane(st.rh.n0, 1);
         const unsigned long long at = lanes_where(st.ol.n[0] == root);
         const int p = at ? __ffsll((long long)at) - 1 : -1;
