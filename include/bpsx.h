@@ -214,7 +214,7 @@ int bpsx_geodesic(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same distances as
  * bpsx_geodesic, but every pointer is a DEVICE pointer, the work is enqueued on hip_stream and
  * the call returns without waiting (out_dist is complete when the stream reaches that point),
- * and the call allocates nothing: its queue, A* node pools and operation logs live in an array of about 4.9 MB
+ * and the call allocates nothing: its queue, A* node pools and operation logs live in an array of about 5.0 MB
  * that each GPU the library runs on holds from library load until the process ends.  At most
  * BPSX_STATIC_MAX_QUERIES queries per call (BPSX_E_INVAL beyond).  All calls on one GPU share
  * that array: calls that overlap on one GPU (other streams, other simulators) race; calls on
