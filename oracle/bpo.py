@@ -64,6 +64,7 @@ class Lib:
             L.bpo_nav_poly_count.argtypes = [C.c_void_p]
             L.bpo_nav_poly_info.argtypes = [C.c_void_p, _u32p, np.ctypeslib.ndpointer(np.uint16), np.ctypeslib.ndpointer(np.int32)]
             L.bpo_nav_last_corridor.argtypes = [C.c_void_p, _u32p, C.c_int]
+            L.bpo_nav_pass_check.argtypes = [C.c_void_p, C.c_int, np.ctypeslib.ndpointer(np.uint64, flags="C_CONTIGUOUS")]
         else:
             L.bpo_nav_find_random_points.argtypes = [C.c_void_p, C.c_uint64, C.c_uint32, _f32p, _u32p]
             L.bpo_ref_create_tile.argtypes = [
@@ -144,6 +145,13 @@ class Nav:
         isl = np.zeros(n, np.int32)
         self.lib.L.bpo_nav_poly_info(self.h, refs, flags, isl)
         return refs, flags, isl
+
+    def pass_check(self, rows):
+        """Switches the check of the GPU kernel's multi-node pass rules (orc::Query::PassCheck) to
+        `rows` nodes per pass (0: off) and returns the counts gathered since the last call."""
+        out = np.zeros(6, np.uint64)
+        self.lib.L.bpo_nav_pass_check(self.h, int(rows), out)
+        return dict(zip(("passes", "nodes", "wrong_node", "wrong_update", "pairs", "ties"), (int(v) for v in out)))
 
     def last_corridor(self):
         buf = np.zeros(256, np.uint32)

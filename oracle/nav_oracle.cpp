@@ -836,7 +836,126 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
     Node* lastBest = startNode;
     float lastBestCost = startNode->total;
     bool outOfNodes = false;
+    // ---- check of the multi-node pass rules (see Query::PassCheck); no effect on the search
+    struct PlanUpd { uint32_t ref; float total; float pos[3]; };
+    struct Plan {
+      int count = 0, done = 0, first = 0;
+      bool pair = false, blind = false;
+      int node[4];
+      std::vector<PlanUpd> upd[4];
+    } plan;
+    auto lookup = [&](uint32_t ref) -> Node* {
+      const uint32_t bucket = Impl::hash(ref) & (HASH_SIZE - 1);
+      for (uint16_t i = q.first[bucket]; i != 0xffff; i = q.next[i])
+        if (q.nodes[i].id == ref) return &q.nodes[i];
+      return nullptr;
+    };
+    // what expanding node `best` writes, computed without changing anything: (polygon, total) in link order
+    auto dry_run = [&](const Node* best, std::vector<uint32_t>& reads, std::vector<PlanUpd>& upds) {
+      const int bestIp = (int)(best->id & ((1u << m.polyBits) - 1));
+      uint32_t parentRef = 0;
+      if (best->pidx) parentRef = q.at(best->pidx)->id;
+      reads.push_back(best->id);
+      for (uint32_t li = m.polys[bestIp].firstLink; li != NULL_LINK; li = m.links[li].next) {
+        const uint32_t nref = m.links[li].ref;
+        if (!nref || nref == parentRef) continue;
+        if (!m.passFilter(m.polys[(int)(nref & ((1u << m.polyBits) - 1))])) continue;
+        reads.push_back(nref);
+        const Node* nn = lookup(nref);
+        float npos[3];
+        uint8_t flags = 0;
+        float ntotal = 0;
+        // a polygon may hold two links to one neighbour: the second sees what the first wrote
+        const PlanUpd* mine = nullptr;
+        for (const PlanUpd& u : upds) if (u.ref == nref) mine = &u;
+        if (nn && nn->flags) { vcopy(npos, nn->pos); flags = nn->flags; ntotal = nn->total; }
+        if (mine) { vcopy(npos, mine->pos); flags = 1; ntotal = mine->total; }
+        if (!flags) {
+          float left[3], right[3];
+          if (!portal_points(m, bestIp, nref, left, right)) continue;
+          for (int k = 0; k < 3; ++k) npos[k] = (left[k] + right[k]) * 0.5f;
+        }
+        float cost, heuristic;
+        if (nref == end.ref) { cost = best->cost + vdist(best->pos, npos) * 1.0f + vdist(npos, end.xyz) * 1.0f; heuristic = 0; }
+        else { cost = best->cost + vdist(best->pos, npos) * 1.0f; heuristic = vdist(npos, end.xyz) * H_SCALE; }
+        const float total = cost + heuristic;
+        if (flags && total >= ntotal) continue;
+        upds.push_back({nref, total, {npos[0], npos[1], npos[2]}});
+      }
+    };
+    auto make_plan = [&]() {
+      plan = Plan();
+      const int rows = (passCheck.rows & 0xff) < 4 ? (passCheck.rows & 0xff) : 4;
+      const bool keyRule = !(passCheck.rows & 0x100), readRule = !(passCheck.rows & 0x200);   // switches for the tests that drop a rule
+      // the open list sorted by total: the first rows + 1 entries
+      std::vector<int> order(q.heapSize);
+      for (int i = 0; i < q.heapSize; ++i) order[i] = q.heap[i];
+      const int want = q.heapSize < rows + 1 ? q.heapSize : rows + 1;
+      std::partial_sort(order.begin(), order.begin() + want, order.end(),
+                        [&](int a, int b) { return q.nodes[a].total < q.nodes[b].total; });
+      const float INF_KEY = std::numeric_limits<float>::infinity();
+      auto key = [&](int j) { return j < q.heapSize ? q.nodes[order[j]].total : INF_KEY; };
+      auto below_next = [&](int j) { return j < q.heapSize && (j + 1 >= q.heapSize || key(j) < key(j + 1)); };
+      int lim = 0;
+      while (lim < rows && below_next(lim)) lim++;
+      if (lim == 0) {
+        // the first two entries share the smallest total: a pair when the third does not
+        if (rows >= 2 && q.heapSize >= 2 && below_next(1)) {
+          plan.pair = true;
+          lim = 2;
+          while (lim < rows && below_next(lim)) lim++;
+        } else { plan.blind = true; plan.count = 1; passCheck.ties++; return; }
+      }
+      for (int j = 0; j < lim; ++j)
+        if (q.nodes[order[j]].id == end.ref) { lim = j == 0 ? 1 : j; break; }
+      if (plan.pair && lim < 2) { plan = Plan(); plan.blind = true; plan.count = 1; passCheck.ties++; return; }
+      std::vector<uint32_t> reads[4];
+      for (int j = 0; j < lim; ++j) {
+        plan.node[j] = order[j];
+        if (q.nodes[order[j]].id != end.ref) dry_run(&q.nodes[order[j]], reads[j], plan.upd[j]);
+      }
+      int c = lim;
+      for (int j = 1; j < c; ++j) {
+        bool stands = true;
+        for (int i = 0; i < j && stands; ++i)
+          for (const PlanUpd& u : plan.upd[i]) {
+            if (keyRule && u.total <= key(j)) { stands = false; break; }
+            if (readRule) for (uint32_t r : reads[j]) if (r == u.ref) { stands = false; break; }
+            if (!stands) break;
+          }
+        if (!stands) { c = j; break; }
+      }
+      if (plan.pair) {
+        bool ok = c >= 2;
+        for (const PlanUpd& u : plan.upd[1]) {
+          if (u.total <= key(1)) ok = false;
+          for (uint32_t r : reads[0]) if (r == u.ref) ok = false;
+        }
+        if (!ok) { plan = Plan(); plan.blind = true; plan.count = 1; passCheck.ties++; return; }
+        passCheck.pairs++;
+      }
+      plan.count = c;
+      passCheck.passes++;
+      passCheck.nodes += (uint64_t)c;
+    };
+    std::vector<PlanUpd> actual;
+    int checking = -1;   // row of the plan whose expansion is under way
     while (q.heapSize > 0) {
+      if (passCheck.rows > 0 && !outOfNodes) {
+        if (plan.done == plan.count) make_plan();
+        checking = -1;
+        if (!plan.blind) {
+          const int top = q.heap[0];
+          int row = plan.done;
+          if (plan.pair && plan.done == 0) row = top == plan.node[1] ? 1 : 0;   // either of the two may come first
+          if (plan.pair && plan.done == 1) row = 1 - plan.first;
+          if (plan.done == 0) plan.first = row;
+          if (top != plan.node[row]) passCheck.wrongNode++;
+          checking = row;
+          actual.clear();
+        }
+        plan.done++;
+      }
       Node* best = q.pop();
       best->flags &= ~NODE_OPEN;
       best->flags |= NODE_CLOSED;
@@ -881,6 +1000,7 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
         nn->flags = (uint8_t)(nn->flags & ~NODE_CLOSED);
         nn->cost = cost;
         nn->total = total;
+        if (checking >= 0) actual.push_back({nref, total, {0, 0, 0}});
         if (nn->flags & NODE_OPEN) {
           q.modify(nn);
         } else {
@@ -888,6 +1008,14 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
           q.push(nn);
         }
         if (heuristic < lastBestCost) { lastBestCost = heuristic; lastBest = nn; }
+      }
+      if (checking >= 0 && !outOfNodes) {
+        // the expansion wrote what the prediction, made from the state before the pass, said
+        const std::vector<PlanUpd>& want = plan.upd[checking];
+        bool same = want.size() == actual.size();
+        for (size_t i = 0; same && i < want.size(); ++i)
+          same = want[i].ref == actual[i].ref && memcmp(&want[i].total, &actual[i].total, 4) == 0;
+        if (!same) passCheck.wrongUpdate++;
       }
     }
     // getPathToNode

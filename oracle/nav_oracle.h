@@ -84,6 +84,20 @@ class Query {
   // has no walkable area.
   bool samplePoint(float u0, float s, float t, float* out_xyz, uint32_t* out_ref);
   Counters counters;
+  // Check of the rules by which the GPU kernel expands several open nodes per pass (TEST
+  // INFRASTRUCTURE like the rest of this file).  With rows > 0, geodesic() predicts before a
+  // pop, from the open list sorted by total and the state as it is, which nodes the next pops
+  // will be and what their expansions will write, by the kernel's rules: entry j stands while its
+  // total is below entry j + 1's, no earlier entry's update reaches its total or touches a
+  // polygon it reads, and it is not the goal; two entries that share the smallest total stand
+  // together, in either order, when neither touches what the other reads.  The search itself is
+  // the reference's, unchanged; every prediction is compared with what it then does.
+  struct PassCheck {
+    int rows = 0;
+    uint64_t passes = 0, nodes = 0;        // predictions made, pops they covered
+    uint64_t wrongNode = 0, wrongUpdate = 0;   // pops of another node / expansions that wrote something else
+    uint64_t pairs = 0, ties = 0;          // tied pairs predicted as a pair / ties left to the heap
+  } passCheck;
 
  private:
   struct Impl;

@@ -97,6 +97,15 @@ BPO_API void bpo_nav_geodesic_field(void* h, const float* sxyz, const uint32_t* 
     out[i] = q.geodesicViaField(a, b);
   }
 }
+// Switches the check of the multi-node pass rules on (rows 1..4) or off (0) for the scene's
+// query object and returns its counts so far: passes, nodes, wrongNode, wrongUpdate, pairs, ties.
+BPO_API void bpo_nav_pass_check(void* h, int rows, uint64_t* out) {
+  orc::Query& q = *((ApiImpl<OracleBackend>::Nav*)h)->ctx->q[0];
+  const orc::Query::PassCheck& p = q.passCheck;
+  out[0] = p.passes; out[1] = p.nodes; out[2] = p.wrongNode; out[3] = p.wrongUpdate; out[4] = p.pairs; out[5] = p.ties;
+  q.passCheck = orc::Query::PassCheck();
+  q.passCheck.rows = rows;
+}
 BPO_API void bpo_random_point_in_convex_poly(const float* pts, int npts, float s, float t, float* out) {
   float areas[16];
   orc::random_point_in_convex_poly(pts, npts, areas, s, t, out);
