@@ -144,7 +144,7 @@ struct HeapEntry {
 // Record of the open-list operations of a search that keeps its open list sorted (see
 // geodesic_device.h): per pass one header (key = number of entries popped | number of records
 // that follow << 8, word = kOpHeader) followed by the pass's pushes and modifies in row and
-// edge order (key = total as bits, word = packed node | row of the pass << 26 | 1 << 28 if the
+// edge order (key = total as bits, word = packed node | row of the pass << 26 | 1 << 29 if the
 // node was open).  A header with kOpUnordered says that the pass's first two rows had the same
 // total: the reference expanded them in the order its heap had them in, which the replay finds
 // out; the header's low 26 bits then name row 0's node.

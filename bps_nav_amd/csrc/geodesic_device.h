@@ -5,8 +5,11 @@
 // Execution model: one wavefront (64 lanes) owns one query at a time and pulls the next from
 // a shared queue when done.  The search touches almost only nodes it created recently (the
 // frontier of A* is narrow), so LDS holds what is hot and small and HBM holds the rest:
-//   - the open list, a binary heap, in registers while it has fewer than 128 entries (entry q
-//     in lane q mod 64); a longer one (rare) keeps its top kHeapLds entries in LDS,
+//   - the open list in registers: sorted by total, up to 256 entries (OpenList), which lets a
+//     pass expand up to kRows nodes at once (astar_fast); the reference's binary heap, also in
+//     registers while it has fewer than 128 entries (RegHeap, entry q in lane q mod 64), is
+//     what a search falls back to when totals tie or the list outgrows its registers; a heap
+//     longer than that (rare) keeps its top kHeapLds entries in LDS,
 //   - the hash heads of the node pool,
 //   - for the first kLinksLds nodes one word with the polygon id, the open/closed flags and the
 //     hash chain link (the parent index is read once per expansion and lives in HBM only),
@@ -29,7 +32,8 @@
 // getEdgeMidPoint); DetourNode.cpp:50-200 (node pool, heap order); PathFinder.cpp:473-541.
 //
 // The sizes of the LDS structures are build parameters (BPSX_LINKS_LDS, BPSX_HEAP_LDS,
-// BPSX_WINDOW, BPSX_HASH), and everything that depends on them lives in namespace
+// BPSX_WINDOW, BPSX_HASH, BPSX_TAG_SLOTS), as is the number of nodes a pass of the sorted-list
+// loop may expand (BPSX_ROWS: 8 rows of 8 lanes, or 4 of 16), and everything that depends on them lives in namespace
 // bpsx::BPSX_GEO_NS (default geo): the file can be included again with other values and
 // another namespace name to get a second instantiation of the same search.
 #include "nav_device.h"
@@ -396,7 +400,7 @@ struct AstarState {
 };
 
 // Applies log records [st.synced, st.logEnd) to the reference's heap, pass by pass.  Records are
-// fetched 64 at a time, one per lane; a pass has at most 1 + 4 * 6 records.  False when the heap
+// fetched 64 at a time, one per lane; a pass has at most 1 + 8 * 6 records.  False when the heap
 // outgrows the registers.
 BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
   RegHeap& rh = st.rh;
@@ -404,7 +408,7 @@ BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
   uint32_t rk = 0, rw = 0;
   bool loaded = false;
   for (int pos = st.synced; pos < st.logEnd;) {
-    if (!loaded || pos + 1 + 4 * kNvp > base + 64) {
+    if (!loaded || pos + 1 + 8 * kNvp > base + 64) {
       base = pos;
       rk = 0; rw = 0;
       if (base + lane < st.logEnd) { const OpRec r = log[base + lane]; rk = r.key; rw = r.word; }
@@ -416,7 +420,7 @@ BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
     // rows in the reference's order: the first two swap when the heap has row 1's node on top
     const bool swap = (hw & kOpUnordered) && rlane(rh.n0, 1) != (hw & 0x3ffffffu);
     const bool mine = lane > h && lane <= h + nrec;
-    const int myRow = (int)((rw >> 26) & 3u);
+    const int myRow = (int)((rw >> 26) & 7u);
     for (int i = 0; i < c; ++i) {
       const int row = (swap && i < 2) ? 1 - i : i;
       rh.pop(lane);
@@ -427,7 +431,7 @@ BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
         const uint32_t key = rlane(rk, j), word = rlane(rw, j);
         const uint32_t node = word & 0x3ffffffu;
         // a node seen as open whose entry has left (its row came earlier in the pass) is pushed
-        int q = ((word >> 28) & 1u) ? rh.position(node, lane) : 0;
+        int q = ((word >> 29) & 1u) ? rh.position(node, lane) : 0;
         if (!q) {
           if (rh.size >= kRegHeap) return false;
           q = ++rh.size;
@@ -463,7 +467,7 @@ namespace bpsx {
 namespace BPSX_GEO_NS {
 
 #ifndef BPSX_LINKS_LDS
-#define BPSX_LINKS_LDS 1144
+#define BPSX_LINKS_LDS 1016
 #endif
 #ifndef BPSX_HEAP_LDS
 #define BPSX_HEAP_LDS 32
@@ -478,8 +482,19 @@ constexpr int kWindow = BPSX_WINDOW;        // most recent nodes whose position/
 #define BPSX_HASH 512
 #endif
 constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash table
-constexpr int kTagSlots = 128;
-constexpr int kRows = 4;                    // nodes expanded per pass of astar_fast, one per row of 16 lanes
+#ifndef BPSX_TAG_SLOTS
+#define BPSX_TAG_SLOTS 256
+#endif
+constexpr int kTagSlots = BPSX_TAG_SLOTS;
+#ifndef BPSX_ROWS
+#define BPSX_ROWS 8
+#endif
+constexpr int kRows = BPSX_ROWS;            // nodes expanded per pass of astar_fast, one per row of 64 / kRows lanes
+constexpr int kRowLanes = 64 / kRows;
+constexpr int kRowShift = kRows == 8 ? 3 : 4;
+static_assert((kRows == 4 || kRows == 8) && kRowLanes > kNvp, "a row needs a lane per edge and one for the node itself");
+// lanes of the rows below j
+constexpr unsigned long long rows_below(int j) { return j * kRowLanes >= 64 ? ~0ull : (1ull << (j * kRowLanes)) - 1ull; }
 static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
 
 // LDS of one wavefront.
@@ -558,7 +573,7 @@ struct GeoWave {
   BPSX_DEV void clear() {
     for (int i = lane; i < kHashSize; i += 64) L->first[i] = (uint16_t)kChainEnd;
     for (int i = lane; i < kTagSlots; i += 64) L->tag[i] = 0xffffffffu;
-    tagNow = 0x3fffffffu;
+    tagNow = 0x1fffffffu;
     heapSize = 0;
     nodeCount = 0;
     wave_sync();
@@ -1051,18 +1066,21 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
 }
 
 // The expansion loop with the open list as a sorted array (OpenList), up to kRows nodes per
-// pass.  Row r of 16 lanes works on entry r of the list (lane 16 r + j on edge j of its
-// polygon): the edge records of all of them arrive in one load, and node lookup, costs, node
+// pass.  Row r of kRowLanes lanes works on entry r of the list (lane kRowLanes r + j on edge j
+// of its polygon, the lane after the last edge on the node itself): the edge records of all of them arrive in one load, and node lookup, costs, node
 // creation and stores are done by the same instructions for all rows.  Every row computes
 // from the state before the pass.  Rows 0 .. c-1 are what the reference does next, in that
 // order, when for every row j below c
 //   - entry j's total is below entry j + 1's, and every total that an earlier row puts on the
 //     open list is above it: entry j is then the only entry with the smallest total when its
 //     turn comes, whatever the arrangement of the reference's heap,
-//   - no earlier row creates or updates a node that row j reads (a neighbour of both, or row
-//     j's own node).  This is found with one LDS word per polygon hash: every lane that
-//     updates notes the pass and its row there (the earliest row wins), every lane then looks
-//     for a note of an earlier row.  Two polygons with the same hash only make c smaller.
+//   - no earlier row creates or updates row j's own node or a node that row j updates too (a
+//     neighbour of both).  A neighbour that row j reads and leaves alone, because the way
+//     through row j is no better than the node's total, may be updated by an earlier row: its
+//     total only gets lower.  This is found with one LDS word per polygon hash: every lane that
+//     updates notes the pass and its row there (the earliest row wins), then these lanes and
+//     the rows' own lanes look for a note of an earlier row.  Two polygons with the same hash
+//     only make c smaller.
 //   - entry j is not the goal (the goal ends the search when it is first in line).
 // The pass commits c >= 1 rows: their new nodes take consecutive indices in row and edge
 // order, their entries leave the list, their updates enter it.  A later row may improve the
@@ -1078,11 +1096,11 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
   endIp = (uint32_t)uniform_i((int)endIp);
   OpenList& ol = st.ol;
-  const int row = lane >> 4, el = lane & 15;
+  const int row = lane >> kRowShift, el = lane & (kRowLanes - 1);
   const bool edgeLane = el < kNvp;
   const bool ownLane = el == kNvp;   // looks after the row's own node in the conflict test
-  constexpr unsigned long long kRowStart = 0x0001000100010001ull;
-  constexpr unsigned long long kRows1 = 0xffffull, kRows2 = 0xffffffffull, kRows3 = 0xffffffffffffull;   // lanes of the first rows
+  constexpr unsigned long long kRowStart = kRows == 8 ? 0x0101010101010101ull : 0x0001000100010001ull;
+  constexpr unsigned long long kRows1 = rows_below(1), kRows2 = rows_below(2);   // lanes of the first rows
   unsigned long long resolved = frontResolved ? 1ull : 0ull;
   // Written for few instructions on the common path: what is rare sits behind one branch each,
   // and conditions that feed a ballot are folded into the compared value first, so that the
@@ -1092,6 +1110,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (!S && g.nodeCount > kLinksLds - kRows * kNvp) return kAstarGrowLinks;
     if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
     FM(0);
+    TIE_WHY(7);   // passes
     // ---- how many entries at the front are each the only one with their total
     const unsigned long long uniq = lanes_where(ol.t[0] < OpenList::down1(OpenList::kEmpty, ol.t[0]));
     int lim = __builtin_ctzll(~uniq | (1ull << kRows));
@@ -1121,7 +1140,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         st.lastBest = biA;
         return kAstarGoal;
       }
-      if (goal) { const int jg = __builtin_ctzll(goal) >> 4; lim = jg < lim ? jg : lim; }
+      if (goal) { const int jg = __builtin_ctzll(goal) >> kRowShift; lim = jg < lim ? jg : lim; }
       if (pairTie && lim < 2) { TIE_WHY(1); return kAstarTie; }   // the goal is one of the two
     }
     FM(1);
@@ -1174,9 +1193,16 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const float cx = p0 - b0, cy = p1 - b1, cz = p2 - b2;
     const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
     const float cc = cx * cx + cy * cy + cz * cz, ee = ex * ex + ey * ey + ez * ez;
-    const float roots = sqrt_exact(lanes_up8(cc, ee));
-    const float curCost = roots * 1.0f;
-    const float toEnd = lanes_down8(roots);
+    float curCost, toEnd;
+    if (kRowLanes == 16) {
+      // both roots in one evaluation: the upper half of a row is idle
+      const float roots = sqrt_exact(lanes_up8(cc, ee));
+      curCost = roots * 1.0f;
+      toEnd = lanes_down8(roots);
+    } else {
+      curCost = sqrt_exact(cc) * 1.0f;
+      toEnd = sqrt_exact(ee);
+    }
     const bool last = nb == endIp;
     const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
     const float heuristic = last ? 0.0f : toEnd * H_SCALE;
@@ -1188,22 +1214,27 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     int c = lim;
     bool pairFails = false;
     if (lim > 1) {
-      const uint32_t k1 = rlane(ol.t[0], 1), k2 = rlane(ol.t[0], 2), k3 = rlane(ol.t[0], 3);
-      const unsigned long long v1 = lanes_where(tb <= k1) & rowsAt1;
-      const unsigned long long v2 = lanes_where(tb <= k2) & kRows2;
-      const unsigned long long v3 = lanes_where(tb <= k3) & kRows3;
-      const int jv = v1 ? 1 : (v2 ? 2 : (v3 ? 3 : 4));
+      // the first entry j that an update of a row before it reaches or undercuts
+      int jv = kRows;
+#pragma unroll
+      for (int j = kRows - 1; j >= 1; --j) {
+        const unsigned long long v = lanes_where(tb <= rlane(ol.t[0], j)) & (j == 1 ? rowsAt1 : rows_below(j));
+        jv = v ? j : jv;
+      }
       c = jv < c ? jv : c;
       // conflicts: the earliest row that updates a polygon leaves its mark (pass, row) at the
       // polygon's hash, later rows look for it: a mark of this pass is base + row
       g.tagNow--;
-      const uint32_t base = g.tagNow << 2;
+      const uint32_t base = g.tagNow << 3;
       const uint32_t slot = bucket & (uint32_t)(kTagSlots - 1);
       if (tb != 0xffffffffu) atomicMin(&L->tag[slot], base | (uint32_t)row);
       wave_sync();
-      const uint32_t seen = L->tag[slot] - base;   // the marking row, or something above 3
-      const uint32_t seenr = (valid || (ownLane && rowOn)) ? seen : 0xffffffffu;
-      const uint32_t jc = (uint32_t)first_lane(lanes_where(seenr < (uint32_t)row)) >> 4;   // none: far above 4
+      const uint32_t seen = L->tag[slot] - base;   // the marking row, or something above 7
+      // an earlier row's update matters to a row only at its own node and at the polygons it
+      // updates itself: where it reads and leaves alone (a total no better than the node's), a
+      // total lowered further changes nothing
+      const uint32_t seenr = (tb != 0xffffffffu || (ownLane && rowOn)) ? seen : 0xffffffffu;
+      const uint32_t jc = (uint32_t)first_lane(lanes_where(seenr < (uint32_t)row)) >> kRowShift;   // none: far above kRows
       c = jc < (uint32_t)c ? (int)jc : c;
       // rows 0 and 1 of a tied pair in either order: row 0 must not read what row 1 updates either
       if (__builtin_expect(pairTie, 0)) {
@@ -1213,13 +1244,13 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
           // The marks are kept per polygon hash, and a pair that fails costs a replay of the log:
           // the polygons that either row updates are compared with those the other row reads,
           // and a clash that was two polygons with one hash lets the pair (and only it) stand.
-          const uint32_t readPoly = ownLane ? (rowOn ? ip : 0xffffffffu) : (valid ? nb : 0xffffffffu);
+          const uint32_t readPoly = ownLane ? (rowOn ? ip : 0xffffffffu) : (tb != 0xffffffffu ? nb : 0xffffffffu);
           unsigned long long w = lanes_where(tb != 0xffffffffu) & kRows2;
           bool real = false;
           while (w) {
             const int src = first_lane(w);
             w = without_lane(w, src);
-            const unsigned long long others = src < 16 ? (kRows2 & ~kRows1) : kRows1;
+            const unsigned long long others = src < kRowLanes ? (kRows2 & ~kRows1) : kRows1;
             if (lanes_where(readPoly == rlane(nb, src)) & others) real = true;
           }
           if (!real) { pairFails = false; c = 2; TIE_WHY(4); } else TIE_WHY(3);
@@ -1294,13 +1325,13 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     {
       // the pass in the operation log: the header from an idle lane, the updates in lane order
       const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(upd >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)upd, 0u));
-      const bool header = lane == 15;
+      const bool header = lane == kRowLanes - 1;   // idle: neither an edge's lane nor the node's own
       const int nrec = __popcll(upd);
       if (update || header) {
         OpRec r;
         r.key = header ? ((uint32_t)c | ((uint32_t)nrec << 8)) : tb;
         r.word = header ? (pairTie ? (kOpHeader | kOpUnordered | rlane(cand, 0)) : kOpHeader)
-                        : (packed | ((uint32_t)row << 26) | ((fl & 1u) << 28));
+                        : (packed | ((uint32_t)row << 26) | ((fl & 1u) << 29));
         g.ws->oplog[st.logEnd + (header ? 0 : 1 + rank)] = r;
       }
       st.logEnd += 1 + nrec;

@@ -841,8 +841,8 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
     struct Plan {
       int count = 0, done = 0, first = 0;
       bool pair = false, blind = false;
-      int node[4];
-      std::vector<PlanUpd> upd[4];
+      int node[8];
+      std::vector<PlanUpd> upd[8];
     } plan;
     auto lookup = [&](uint32_t ref) -> Node* {
       const uint32_t bucket = Impl::hash(ref) & (HASH_SIZE - 1);
@@ -885,7 +885,7 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
     };
     auto make_plan = [&]() {
       plan = Plan();
-      const int rows = (passCheck.rows & 0xff) < 4 ? (passCheck.rows & 0xff) : 4;
+      const int rows = (passCheck.rows & 0xff) < 8 ? (passCheck.rows & 0xff) : 8;
       const bool keyRule = !(passCheck.rows & 0x100), readRule = !(passCheck.rows & 0x200);   // switches for the tests that drop a rule
       // the open list sorted by total: the first rows + 1 entries
       std::vector<int> order(q.heapSize);
@@ -909,10 +909,16 @@ float Query::geodesic(const NavPoint& start, const NavPoint& end) {
       for (int j = 0; j < lim; ++j)
         if (q.nodes[order[j]].id == end.ref) { lim = j == 0 ? 1 : j; break; }
       if (plan.pair && lim < 2) { plan = Plan(); plan.blind = true; plan.count = 1; passCheck.ties++; return; }
-      std::vector<uint32_t> reads[4];
+      std::vector<uint32_t> reads[8];
       for (int j = 0; j < lim; ++j) {
         plan.node[j] = order[j];
         if (q.nodes[order[j]].id != end.ref) dry_run(&q.nodes[order[j]], reads[j], plan.upd[j]);
+      }
+      // a row depends on an earlier update only through its own node and through the polygons
+      // that it updates itself: what it reads and leaves alone only gets a lower total
+      for (int j = 0; j < lim; ++j) {
+        reads[j].assign(1, q.nodes[order[j]].id);
+        for (const PlanUpd& u : plan.upd[j]) reads[j].push_back(u.ref);
       }
       int c = lim;
       for (int j = 1; j < c; ++j) {

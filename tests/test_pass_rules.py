@@ -23,7 +23,7 @@ def test_predicted_passes_are_what_the_reference_does(oracle, config, queries):
     x, r = x[ok], r[ok]
     m = len(x) // 2
     plain = nav.geodesic(x[:m], r[:m], x[m:2 * m], r[m:2 * m])
-    nav.pass_check(4)
+    nav.pass_check(8)
     checked = nav.geodesic(x[:m], r[:m], x[m:2 * m], r[m:2 * m])
     st = nav.pass_check(0)
     nav.close()
@@ -58,7 +58,7 @@ def test_each_rule_is_needed(oracle, dropped, what):
     nav = bpo.Nav(oracle, blob)
     pts = scenes.sample_points(blob, 11, 400)
     x, r = nav.snap(pts)
-    nav.pass_check(4 | dropped)
+    nav.pass_check(8 | dropped)
     nav.geodesic(x[:200], r[:200], x[200:], r[200:])
     st = nav.pass_check(0)
     nav.close()
