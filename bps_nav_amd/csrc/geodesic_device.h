@@ -1118,7 +1118,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const int bi = (int)(cand & 0x7ffu);
     const uint32_t ip = cand >> 11;
     const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
-    bool pairTie = false;
+    bool pairTie = false, goalInPair = false;
     unsigned long long rowsAt1 = kRows1;   // rows whose updates must lie above entry 1's total
     if (__builtin_expect((goal | ((uniq & 1ull) ^ 1ull) | resolved) != 0, 0)) {
       if (resolved) { lim = 1; resolved = 0; }   // the caller has put the reference's next node first
@@ -1134,14 +1134,15 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         rowsAt1 = kRows2;
         lim = __builtin_ctzll(~(uniq | 3ull) | (1ull << kRows));
       }
-      if (goal & 1ull) {
+      if ((goal & 1ull) && !pairTie) {
         const int biA = uniform_i(bi);
         g.set_link<S>(biA, with_flags(g.link<S>(biA), 2u));
         st.lastBest = biA;
         return kAstarGoal;
       }
-      if (goal) { const int jg = __builtin_ctzll(goal) >> kRowShift; lim = jg < lim ? jg : lim; }
-      if (pairTie && lim < 2) { TIE_WHY(1); return kAstarTie; }   // the goal is one of the two
+      // the goal as one of a tied pair: both rows are looked at, the goal's row without its edges
+      if (pairTie && (goal & kRows2)) { goalInPair = true; lim = 2; }
+      else if (goal) { const int jg = __builtin_ctzll(goal) >> kRowShift; lim = jg < lim ? jg : lim; }
     }
     FM(1);
     const bool rowOn = row < lim;
@@ -1152,6 +1153,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       const AEdge e = edges[ip * kEdgeStride + (uint32_t)el];
       nb = e.nb; m0 = e.mid[0]; m1 = e.mid[1]; m2 = e.mid[2];
     }
+    if (__builtin_expect(goalInPair, 0)) nb = ip == endIp ? kNoNb : nb;
     const int bis = rowOn ? bi : 0;
     const uint32_t blink = g.link<S>(bis);
     float b0, b1, b2, bcost;
@@ -1210,6 +1212,20 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     // the total as bits where the lane updates its node, all ones where it does not
     uint32_t tb = (valid && !(fl && total >= oldTotal)) ? __float_as_uint(total) : 0xffffffffu;
     FM(4);
+    if (__builtin_expect(goalInPair, 0)) {
+      // The goal shares the smallest total with one other node.  If the reference takes the goal
+      // first the search ends here; if it takes the other node first, it expands it and ends
+      // then.  The path is the goal's node and its ancestors: it is the same both ways when
+      // that expansion only creates nodes (none of them can be on the path) and the node pool
+      // holds them (an exhausted pool is reported as failure).  Otherwise the heap must say.
+      const unsigned long long touches = lanes_where(tb != 0xffffffffu && ni >= 0);
+      const int fresh = __popcll(lanes_where(tb != 0xffffffffu));
+      if (touches || g.nodeCount + fresh > kMaxNodes) { TIE_WHY(1); return kAstarTie; }
+      const int biG = (int)rlane((uint32_t)bi, first_lane(goal & kRows2));
+      g.set_link<S>(biG, with_flags(g.link<S>(biG), 2u));
+      st.lastBest = biG;
+      return kAstarGoal;
+    }
     // ---- how many rows stand
     int c = lim;
     bool pairFails = false;
@@ -1433,6 +1449,7 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         // mazes and rooms, both in a hall without obstacles): the search runs again with the exact loops
         if (ex == kAstarGrowHeap || ex == kAstarLogFull) { restart = true; break; }
         if (ex != kAstarTie) break;
+        __builtin_amdgcn_s_setprio(3);   // a search that pays for a replay is late from here on
         // a tie: the reference pops what its heap has at the root, so the heap is brought up to
         // date from the log, and that entry goes first
 #ifdef BPSX_TIE_REASONS
