@@ -400,20 +400,22 @@ struct AstarState {
 };
 
 // Applies log records [st.synced, st.logEnd) to the reference's heap, pass by pass.  Records are
-// fetched 64 at a time, one per lane; a pass has at most 1 + 8 * 6 records.  False when the heap
+// fetched 64 at a time, one per lane, and again when the next pass is not among them in full
+// (a pass has at most 1 + 8 * 6 records).  False when the heap
 // outgrows the registers.
 BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
   RegHeap& rh = st.rh;
-  int base = st.synced;        // record held by lane 0
+  int base = -64;              // record held by lane 0
   uint32_t rk = 0, rw = 0;
-  bool loaded = false;
+  auto fetch = [&](int from) {
+    base = from;
+    rk = 0; rw = 0;
+    if (base + lane < st.logEnd) { const OpRec r = log[base + lane]; rk = r.key; rw = r.word; }
+  };
   for (int pos = st.synced; pos < st.logEnd;) {
-    if (!loaded || pos + 1 + 8 * kNvp > base + 64) {
-      base = pos;
-      rk = 0; rw = 0;
-      if (base + lane < st.logEnd) { const OpRec r = log[base + lane]; rk = r.key; rw = r.word; }
-      loaded = true;
-    }
+    // a fetch is a round trip to HBM: one only when the pass at hand is not all there
+    if (pos >= base + 64) fetch(pos);
+    if (pos - base + 1 + (int)(rlane(rk, pos - base) >> 8) > 64) fetch(pos);
     const int h = pos - base;
     const uint32_t hk = rlane(rk, h), hw = rlane(rw, h);
     const int c = (int)(hk & 0xffu), nrec = (int)(hk >> 8);
