@@ -448,6 +448,23 @@ BPSX_DEV bool replay_log(const OpRec* log, AstarState& st, int lane) {
 }
 enum AstarExit { kAstarEmpty = 0, kAstarGoal = 1, kAstarGrowLinks = 2, kAstarGrowHeap = 3, kAstarTie = 4, kAstarLogFull = 5 };
 
+// Two roots at once: one test of the arguments' range for both.
+BPSX_DEV void sqrt_exact2(float x, float y, float* rx, float* ry) {
+  const uint32_t xb = __float_as_uint(x), yb = __float_as_uint(y);
+  if (__builtin_expect(lanes_where(xb - 1u < 0x0f800000u - 1u || yb - 1u < 0x0f800000u - 1u) != 0, 0)) {
+    *rx = sqrtf(x); *ry = sqrtf(y);   // 0 < argument < 2^-96 in some lane: never in practice
+    return;
+  }
+  const float s = __builtin_amdgcn_sqrtf(x), t = __builtin_amdgcn_sqrtf(y);
+  const float sd = __uint_as_float(__float_as_uint(s) - 1u), su = __uint_as_float(__float_as_uint(s) + 1u);
+  const float td = __uint_as_float(__float_as_uint(t) - 1u), tu = __uint_as_float(__float_as_uint(t) + 1u);
+  float r = fmaf(-sd, s, x) <= 0.0f ? sd : s;
+  r = fmaf(-su, s, x) > 0.0f ? su : r;
+  float q = fmaf(-td, t, y) <= 0.0f ? td : t;
+  q = fmaf(-tu, t, y) > 0.0f ? tu : q;
+  *rx = r; *ry = q;
+}
+
 BPSX_DEV float tri_area2d(const float* a, const float* b, const float* c) {
   const float abx = b[0] - a[0], abz = b[2] - a[2];
   const float acx = c[0] - a[0], acz = c[2] - a[2];
@@ -1204,8 +1221,8 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       curCost = roots * 1.0f;
       toEnd = lanes_down8(roots);
     } else {
-      curCost = sqrt_exact(cc) * 1.0f;
-      toEnd = sqrt_exact(ee);
+      sqrt_exact2(cc, ee, &curCost, &toEnd);
+      curCost = curCost * 1.0f;
     }
     const bool last = nb == endIp;
     const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
