@@ -532,7 +532,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   static_assert(kHalf % 16 == 0 && sizeof(geo_long::GeoShared) <= 2 * kHalf, "the long search must fit the LDS of one block");
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kHalf];
   __shared__ uint32_t long_ticket;
-  const int lane = (int)(threadIdx.x & 63), half = (int)(threadIdx.x >> 6);
+  const int lane = (int)(threadIdx.x & 63), half = uniform_i((int)(threadIdx.x >> 6));   // the same in all lanes, and known to be: addresses derived from it stay in scalar registers
   GeoSlot* slot = &slots[blockIdx.x * 2 + half];
   // classes are served in order: class c owns ticket numbers [first[c], first[c + 1])
   uint32_t first[kGeoClasses + 1];
