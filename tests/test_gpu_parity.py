@@ -84,6 +84,31 @@ def test_batched_queries_match_oracle(oracle, torch_cuda, config):
     gen.close()
 
 
+@pytest.mark.parametrize("config,seed", [(1, 101), (2, 100), (2, 103), (3, 100), (4, 101), (4, 104)])
+def test_geodesics_on_further_scenes_match_oracle(oracle, torch_cuda, config, seed):
+    """Scene-wide point pairs on generated scenes that no other test uses: the searches meet other
+    junctions, equal totals and pool sizes than those of the scenes above."""
+    from bps_nav_amd import scenes
+    from bps_nav_amd.bps_sim import nav_only
+    from oracle import bpo
+    print(f"case: geodesics on config {config} scene {seed}", flush=True)
+    blob = scenes.config_scene(config, seed)
+    nav = bpo.Nav(oracle, blob)
+    gen = nav_only([blob])
+    pts = scenes.sample_points(blob, 1000 + seed, 3000)
+    x, r = nav.snap(pts)
+    ok = r != 0
+    x, r = x[ok], r[ok]
+    m = len(x) // 2
+    go = nav.geodesic(x[:m], r[:m], x[m:2 * m], r[m:2 * m])
+    gg = gen.geodesic(0, x[:m], r[:m], x[m:2 * m], r[m:2 * m])
+    nav.close()
+    assert m > 1000 and np.isfinite(go).sum() > 100   # (maze-wide pairs mostly exceed the 256-polygon path limit: +inf on both sides)
+    assert np.array_equal(common.bits(go), common.bits(gg)), \
+        f"{(common.bits(go) != common.bits(gg)).sum()} of {m} geodesics differ"
+    gen.close()
+
+
 @pytest.mark.parametrize("name", ["recast_room", "recast_two_floors"])
 def test_recast_built_meshes_match_reference_vectors(oracle, torch_cuda, name):
     """Navmeshes built by the reference's own Recast (committed fixtures): the engine against the
