@@ -36,7 +36,11 @@ namespace {
 const char* const kKernelNames[BPSX_NUM_KERNELS] = {"step_move", "reset_snap", "geodesic", "step_finish"};
 
 struct Group {
-  StepQueues Q{};
+  // Two sets of queues, used in turn: a step's launch serves Q[turn] and puts the first queries
+  // of the episodes that begin in it into the other set, which the next step serves.
+  StepQueues Q[2] = {};
+  int turn = 0;
+  hipEvent_t moved = nullptr, snapped = nullptr;   // fork and join of the side stream within a step
   int64_t* d_actions = nullptr;
   int64_t* h_actions = nullptr;  // pinned staging for host-side action arrays
   hipEvent_t done = nullptr;
@@ -176,6 +180,7 @@ struct bpsx_sim {
   bool loader_exit = false;
   std::string loader_error;              // first failure of the loader thread (guarded by loader_mu)
   hipStream_t upload_stream = nullptr;   // uploads of scenes that come in while the simulation runs
+  hipStream_t side = nullptr;            // a step's snaps of new episodes, next to its searches (default priority)
   uint32_t* h_swap_remaining = nullptr;  // pinned copy of d_swap_remaining, refreshed by every step
   bool remaining_fresh = false;
   std::vector<uint32_t> rotation_log;    // (step ordinal, slot, dataset index) of swaps made available
@@ -475,6 +480,7 @@ int bpsx_finalize(bpsx_sim* sim) {
     HIP_TRY(hipMemcpy(sim->d_swap_target, none.data(), (size_t)S * 4, hipMemcpyHostToDevice));
   }
   HIP_TRY(hipStreamCreateWithFlags(&sim->upload_stream, hipStreamNonBlocking));
+  HIP_TRY(hipStreamCreateWithFlags(&sim->side, hipStreamNonBlocking));
   HIP_TRY(hipHostMalloc((void**)&sim->h_swap_remaining, (size_t)S * 4, hipHostMallocDefault));
   memset(sim->h_swap_remaining, 0, (size_t)S * 4);
   for (uint32_t i = 0; i < S; ++i) {
@@ -533,10 +539,15 @@ int bpsx_finalize(bpsx_sim* sim) {
   sim->groups.resize(sim->num_groups);
   const size_t n = sim->envs_per_group;
   for (auto& g : sim->groups) {
-    if ((rc = sim->alloc(&g.Q.counts, kQCounters)) || (rc = sim->alloc(&g.Q.queries, (size_t)kGeoClasses * 2 * n)) ||
-        (rc = sim->alloc(&g.Q.reset_list, n)) || (rc = sim->alloc(&g.d_actions, n)))
-      return rc;
-    g.Q.stride = (uint32_t)(2 * n);
+    for (StepQueues& Q : g.Q) {
+      if ((rc = sim->alloc(&Q.counts, kQCounters)) || (rc = sim->alloc(&Q.queries, (size_t)kGeoClasses * 2 * n)) ||
+          (rc = sim->alloc(&Q.reset_list, n)))
+        return rc;
+      Q.stride = (uint32_t)(2 * n);
+    }
+    if ((rc = sim->alloc(&g.d_actions, n))) return rc;
+    HIP_TRY(hipEventCreateWithFlags(&g.moved, hipEventDisableTiming));
+    HIP_TRY(hipEventCreateWithFlags(&g.snapped, hipEventDisableTiming));
     HIP_TRY(hipHostMalloc((void**)&g.h_actions, n * sizeof(int64_t), hipHostMallocDefault));
     HIP_TRY(hipEventCreateWithFlags(&g.done, hipEventDisableTiming));
     for (auto& e : g.ev) HIP_TRY(hipEventCreate(&e));
@@ -568,10 +579,13 @@ void bpsx_destroy(bpsx_sim* sim) {
     sim->loader.join();
   }
   if (sim->upload_stream) (void)hipStreamDestroy(sim->upload_stream);
+  if (sim->side) (void)hipStreamDestroy(sim->side);
   if (sim->h_swap_remaining) (void)hipHostFree(sim->h_swap_remaining);
   for (auto& g : sim->groups) {
     if (g.h_actions) (void)hipHostFree(g.h_actions);
     if (g.done) (void)hipEventDestroy(g.done);
+    if (g.moved) (void)hipEventDestroy(g.moved);
+    if (g.snapped) (void)hipEventDestroy(g.snapped);
     for (auto& e : g.ev)
       if (e) (void)hipEventDestroy(e);
   }
@@ -600,7 +614,7 @@ int bpsx_reset(bpsx_sim* sim, uint32_t group, void* hip_stream) {
   if (g.in_flight) return fail(BPSX_E_STATE, "reset: a step of this group is still in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
   hipStream_t st = (hipStream_t)hip_stream;
-  launch_reset(sim->nav, sim->A, g.Q, sim->params(group), sim->d_slots, sim->geo_blocks, sim->snap_blocks, st);
+  launch_reset(sim->nav, sim->A, g.Q[g.turn], g.Q[g.turn ^ 1], sim->params(group), sim->d_slots, sim->geo_blocks, sim->snap_blocks, st);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipStreamSynchronize(st));
   return BPSX_OK;
@@ -624,8 +638,11 @@ int bpsx_step_start(bpsx_sim* sim, uint32_t group, const int64_t* actions, int a
   }
   if ((rc = rotation_pre_step(sim, st))) return rc;
   g.profiled = sim->profiling;
-  launch_step(sim->nav, sim->A, g.Q, sim->params(group), d_act, sim->d_slots, sim->geo_blocks, sim->snap_blocks, st,
-              g.profiled ? g.ev : nullptr);
+  StepParams P = sim->params(group);
+  P.defer_first_distance = 1;
+  launch_step(sim->nav, sim->A, g.Q[g.turn], g.Q[g.turn ^ 1], P, d_act, sim->d_slots, sim->geo_blocks, sim->snap_blocks, st,
+              sim->side, g.moved, g.snapped, g.profiled ? g.ev : nullptr);
+  g.turn ^= 1;
   HIP_TRY(hipGetLastError());
   // how many envs of each slot are still on a scene that is leaving: read back with the step
   sim->remaining_fresh = false;

@@ -33,16 +33,24 @@ struct StepParams {
   uint32_t num_slots;
   const uint32_t* swap_target;
   uint32_t* swap_remaining;
+  // 1: the first distance of an episode that begins in this step is measured in the next step's
+  // launch (see launch_step); 0: in this one
+  uint32_t defer_first_distance;
 };
 constexpr uint32_t kNoSwap = 0xffffffffu;
 
 constexpr int kStepEvents = 5;  // timestamps recorded by launch_step when asked to
 
-void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
+// One step of a group.  Q holds the step's queries, among them the first queries of the episodes
+// that began in the previous step; the episodes that begin in this one are snapped on `side`
+// while the searches run on `st`, and their first queries go to Qnext, the next step's queues.
+// `moved` and `snapped` are events of the caller's for the fork and the join of the two streams.
+void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepQueues& Qnext, const StepParams& P,
                  const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st,
-                 hipEvent_t* ev);
-void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P, GeoSlot* slots,
-                  uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st);
+                 hipStream_t side, hipEvent_t moved, hipEvent_t snapped, hipEvent_t* ev);
+// Reset of a whole group, all on st; Qother (the group's other set of queues) is emptied.
+void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepQueues& Qother, const StepParams& P,
+                  GeoSlot* slots, uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st);
 void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref,
                        uint32_t snap_blocks, hipStream_t st);
 void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,

@@ -1,6 +1,6 @@
 // HIP kernels of the batch environment step (gfx950) and their launch wrappers.
 //
-// One step of a group of n agents is four launches on one stream:
+// One step of a group of n agents is four launches:
 //   step_move      lane per agent: action, turn / forward move with wall sliding, polar
 //                  observation, and a geodesic query (goal -> agent) when the agent moved or
 //                  the episode ended; an agent whose episode ended also picks its next episode
@@ -13,6 +13,11 @@
 //                                                        (PathFinder.cpp:485-541)
 //   step_finish    lane per agent: info, reward, mask from the terminal transition, then the
 //                  new episode's distance bookkeeping    (simulator.cpp:634-641, 758-822, 749-755)
+// In a step, reset_snap runs on a second stream next to geodesic: the first query of an episode
+// that begins in step t is answered by step t + 1's geodesic launch, and its result enters the
+// bookkeeping at the start of step t + 1's step_finish.  No output of step t depends on it (the
+// reference computes it inside the reset and uses it from the next step on).  A reset of a
+// whole group (bpsx_reset) runs the four launches in order, first queries included.
 // The Flee and Exploration tasks (simulator.cpp:830-997) run through the same four launches:
 // Flee keeps the episode's start point where PointNav keeps the snapped goal, so its
 // "distance from start" is the same start-point -> agent query; Exploration makes no queries
@@ -139,10 +144,13 @@ __global__ void k_set_swap(uint32_t* swap_target, uint32_t* swap_remaining, uint
   }
 }
 
-__global__ void k_clear_queues(StepQueues Q) {
+// Empties all of Q, and the reset list and the ticket counters of R (which may be Q again): R's
+// lists of queries may already hold what an earlier launch has put there for the coming one.
+__global__ void k_clear_queues(StepQueues Q, StepQueues R) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     for (int c = 0; c < kGeoClasses; ++c) Q.counts[kQGeo + c] = 0;
     Q.counts[kQGeoHead] = 0; Q.counts[kQGeoHeadLong] = 0; Q.counts[kQReset] = 0;
+    R.counts[kQGeoHead] = 0; R.counts[kQGeoHeadLong] = 0; R.counts[kQReset] = 0;
   }
 }
 
@@ -206,7 +214,7 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
       uint32_t navRefNow = A.nav_ref[gi];
       load3(A.goal_xyz, gi, goalNav);
       const uint32_t goalRef = A.goal_ref[gi];
-      const bool distOk = A.dist_ok[gi] != 0;
+      const bool distOk = A.dist_ok[gi] == 1;
       const uint32_t expected = A.last_cost[gi];
       A.step[gi] = step;
       bool done = (float)step >= P.max_steps;
@@ -344,6 +352,14 @@ __global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P
     }
     return;
   }
+  if (A.dist_ok[gi] == 2) {
+    // the episode began in the previous step: its first distance has been measured in this one
+    const float d = A.geo[(size_t)P.total + gi];
+    A.init[gi] = d;
+    A.info_prev[gi] = d;   // agent->goal: not a goal->agent result, so not reusable
+    A.rew_prev[gi] = d;
+    A.dist_ok[gi] = 0;
+  }
   if (!(f & kAgentResetOnly)) {
     float dist, success = 0, spl = 0;
     const float fresh = (f & kAgentReuse) ? A.info_prev[gi] : A.geo[gi];
@@ -377,13 +393,18 @@ __global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P
     A.infos[(size_t)gi * 3 + 2] = dist;
   }
   if (done || (f & kAgentResetOnly)) {
-    // InfoFunctor::reset / RewardFunctor::reset with the new episode's first distance
-    const float d = A.geo[(size_t)P.total + gi];
+    // InfoFunctor::reset / RewardFunctor::reset with the new episode's first distance, which a
+    // step leaves to the next step's launch (no output of this step depends on it)
     A.cum[gi] = 0;
-    A.init[gi] = d;
-    A.info_prev[gi] = d;   // agent->goal: not a goal->agent result, so not reusable
-    A.dist_ok[gi] = 0;
-    A.rew_prev[gi] = d;
+    if (P.defer_first_distance && !(f & kAgentResetOnly)) {
+      A.dist_ok[gi] = 2;
+    } else {
+      const float d = A.geo[(size_t)P.total + gi];
+      A.init[gi] = d;
+      A.info_prev[gi] = d;   // agent->goal: not a goal->agent result, so not reusable
+      A.dist_ok[gi] = 0;
+      A.rew_prev[gi] = d;
+    }
     float pos[3];
     load3(A.pos, gi, pos);
     store3(A.prev_pos, gi, pos);
@@ -403,7 +424,7 @@ __global__ __launch_bounds__(256) void k_reset_all(NavData nav, AgentArrays A, S
 // One block of two wavefronts per agent being reset: each takes one snap of the new episode (the
 // two are independent chains of dependent loads), then the first writes the state, the polar
 // observation and the episode's first geodesic query.
-__global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, StepQueues Q, StepParams P) {
+__global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, StepQueues Q, StepQueues Qout, StepParams P) {
   __shared__ SnapLds lds[2];
   __shared__ NavPt goalPt;
   const uint32_t n = Q.counts[kQReset];
@@ -460,7 +481,7 @@ __global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, 
       q.cost_slot = kNoCostSlot;   // searched agent -> goal: says little about the searches to come
       q.pad = 0;
       // a new episode: no history
-      Q.queries[(size_t)kGeoClassUnknown * Q.stride + atomicAdd(&Q.counts[kQGeo + kGeoClassUnknown], 1u)] = q;
+      Qout.queries[(size_t)kGeoClassUnknown * Qout.stride + atomicAdd(&Qout.counts[kQGeo + kGeoClassUnknown], 1u)] = q;
     }
     __syncthreads();   // goalPt is rewritten in the next round
   }
@@ -673,29 +694,42 @@ void launch_geodesic(const NavData& nav, const GeoQuery* queries, uint32_t strid
                      last_cost, slots, counters);
 }
 
-void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P,
+void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepQueues& Qnext, const StepParams& P,
                  const int64_t* actions_dev, GeoSlot* slots, uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st,
-                 hipEvent_t* ev) {
+                 hipStream_t side, hipEvent_t moved, hipEvent_t snapped, hipEvent_t* ev) {
   int e = 0;
   auto mark = [&]() { if (ev) (void)hipEventRecord(ev[e++], st); };
   mark();
-  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
+  // Q's lists of queries were emptied a step ago and have since taken the first queries of the
+  // episodes that began in the previous step; its reset list is emptied now, and so is Qnext
+  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Qnext, Q);
   hipLaunchKernelGGL(k_step_move, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P, actions_dev);
   mark();
-  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, P);
+  // the new episodes' snaps need nothing of this step's searches and the searches nothing of
+  // them: they run side by side
+  // (not when the launches are being timed one by one: then everything stays on st)
+  const bool fork = side && !ev;
+  if (fork) {
+    (void)hipEventRecord(moved, st);
+    (void)hipStreamWaitEvent(side, moved, 0);
+  }
+  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, fork ? side : st, nav, A, Q, Qnext, P);
+  if (fork) (void)hipEventRecord(snapped, side);
   mark();
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
   mark();
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
+  if (fork) (void)hipStreamWaitEvent(st, snapped, 0);
   mark();
 }
 
-void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepParams& P, GeoSlot* slots,
-                  uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st) {
-  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q);
+void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q, const StepQueues& Qother, const StepParams& P,
+                  GeoSlot* slots, uint32_t geo_blocks, uint32_t snap_blocks, hipStream_t st) {
+  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q, Qother);
+  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Qother, Qother);
   hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
-  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, P);
+  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, Q, P);
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);

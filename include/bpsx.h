@@ -158,7 +158,12 @@ int bpsx_num_groups(const bpsx_sim *sim, uint32_t *out);
 int bpsx_reset(bpsx_sim *sim, uint32_t group, void *hip_stream);
 /* step_start(group, actions): actions int64[n] in {0 stop, 1 forward, 2 left, 3 right};
  * actions_on_device != 0 => device pointer (read in stream order), else host pointer
- * (copied before returning).  Enqueues the step; returns without waiting. */
+ * (copied before returning).  Enqueues the step; returns without waiting.  Part of the step
+ * (the snaps of the episodes that begin in it) runs on a stream of the library's own, forked
+ * from and joined to hip_stream with events: work enqueued on hip_stream afterwards sees the
+ * whole step.  The first distance of an episode that begins in a step is measured by the next
+ * step (the reference measures it at once, simulator.cpp:744-751, and uses it from the next
+ * step on): outputs and state arrays are the same after every step. */
 int bpsx_step_start(bpsx_sim *sim, uint32_t group, const int64_t *actions,
                     int actions_on_device, void *hip_stream);
 /* step_end(group): waits until the step's outputs are complete. */
