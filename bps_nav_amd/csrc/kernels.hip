@@ -24,6 +24,8 @@
 // and keeps its visited cells per agent in HBM.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "../../include/bpsx.h"
 #include "geodesic_device.h"
 // A second instantiation of the same search for the few longest queries of a step: all 2048
@@ -713,7 +715,10 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
     (void)hipEventRecord(moved, st);
     (void)hipStreamWaitEvent(side, moved, 0);
   }
-  hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, fork ? side : st, nav, A, Q, Qnext, P);
+  // (a grid for one agent in sixteen ending its episode; more take further rounds.  Blocks
+  // without work would only wait for LDS that the searches hold and keep the join waiting.)
+  const uint32_t step_snap_blocks = std::min(snap_blocks, std::max(64u, P.n / 16u));
+  hipLaunchKernelGGL(k_reset_snap, dim3(step_snap_blocks), dim3(128), 0, fork ? side : st, nav, A, Q, Qnext, P);
   if (fork) (void)hipEventRecord(snapped, side);
   mark();
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
@@ -733,6 +738,8 @@ void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q,
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
+  // the next step finds its lists of queries empty, not with this launch's queries still in them
+  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q, Q);
 }
 
 void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uint32_t n, float* oxyz, uint32_t* oref,
