@@ -6,7 +6,7 @@
 
 namespace bpsx {
 
-enum QueueCounter { kQGeo = 0 /* one per cost class */, kQGeoHead = kGeoClasses, kQReset, kQGeoHeadLong, kQCounters };
+enum QueueCounter { kQGeo = 0 /* one per cost class */, kQGeoHead = kGeoClasses, kQReset, kQCounters };
 
 // Work queues of one step, all in HBM, sized for every agent of a group.
 struct StepQueues {
@@ -56,7 +56,7 @@ void launch_snap_batch(const NavData& nav, uint32_t scene, const float* pts, uin
 void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
                            uint32_t n, float* oxyz, uint32_t* oref, hipStream_t st);
 void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
-                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 2] */,
+                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 1] */,
                            float* out,
                            GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st);
 void launch_random_points(const NavData& nav, uint32_t scene, const float* u, uint32_t n, float* oxyz, uint32_t* oref,

@@ -151,8 +151,8 @@ __global__ void k_set_swap(uint32_t* swap_target, uint32_t* swap_remaining, uint
 __global__ void k_clear_queues(StepQueues Q, StepQueues R) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     for (int c = 0; c < kGeoClasses; ++c) Q.counts[kQGeo + c] = 0;
-    Q.counts[kQGeoHead] = 0; Q.counts[kQGeoHeadLong] = 0; Q.counts[kQReset] = 0;
-    R.counts[kQGeoHead] = 0; R.counts[kQGeoHeadLong] = 0; R.counts[kQReset] = 0;
+    Q.counts[kQGeoHead] = 0; Q.counts[kQReset] = 0;
+    R.counts[kQGeoHead] = 0; R.counts[kQReset] = 0;
   }
 }
 
@@ -543,18 +543,18 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
 
 // Blocks of two wavefronts, each wavefront persistent and serving queries from the shared
 // queue on its half of the block's LDS.  The launch ends with its longest search, so the
-// queries of the kLongClasses longest classes are treated apart: at its start the first
-// wavefront of every block draws a ticket for one of them, and a block that gets one gives it
-// the whole block's LDS (the larger instantiation: no link spills, half the window misses,
-// shorter hash chains; 7 % faster on such searches) while its second wavefront leaves.
+// queries of the kLongClasses longest classes are treated apart: block b takes the b-th of
+// them, if there is one, and gives it the whole block's LDS (the larger instantiation: no link
+// spills, half the window misses, shorter hash chains; 7 % faster on such searches) while its
+// second wavefront leaves.  Every other wavefront's first query is fixed by its index too;
+// from the second query on a wavefront draws from the queue's counter.
 constexpr int kLongClasses = 2;   // expected cost of 1400 nodes and more
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
-                                                  const uint32_t* __restrict__ counts, uint32_t* head, uint32_t* head_long,
+                                                  const uint32_t* __restrict__ counts, uint32_t* head,
                                                   float* out, uint32_t* last_cost, GeoSlot* slots, uint64_t* counters) {
   constexpr size_t kHalf = sizeof(geo::GeoShared);
   static_assert(kHalf % 16 == 0 && sizeof(geo_long::GeoShared) <= 2 * kHalf, "the long search must fit the LDS of one block");
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kHalf];
-  __shared__ uint32_t long_ticket;
   const int lane = (int)(threadIdx.x & 63), half = uniform_i((int)(threadIdx.x >> 6));   // the same in all lanes, and known to be: addresses derived from it stay in scalar registers
   GeoSlot* slot = &slots[blockIdx.x * 2 + half];
   // classes are served in order: class c owns ticket numbers [first[c], first[c + 1])
@@ -564,9 +564,11 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   const uint32_t nq = first[kGeoClasses], nlong = first[kLongClasses];
   GeoTotals T;
   uint32_t linkSpills = 0, heapSpills = 0, exactRuns = 0, tieReplays = 0, pairTies = 0;
-  if (threadIdx.x == 0) long_ticket = atomicAdd(head_long, 1u);
-  __syncthreads();
-  const uint32_t lt = (uint32_t)uniform_i((int)long_ticket);
+  // The first query of every wavefront needs no ticket counter: the grid is what the device
+  // holds at once, so block b takes long query b if there is one, and the wavefronts of the
+  // other blocks take the queries after the long ones in the order of their index.  (Some
+  // thousand atomics on one counter at the start of a launch are served one after the other.)
+  const uint32_t lt = blockIdx.x;
   if (lt < nlong) {
     if (half == 1) return;
     geo_long::GeoWave gl;
@@ -598,12 +600,18 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
 #endif
   // tickets below `taken` went to the blocks' first wavefronts above
   const uint32_t taken = nlong < gridDim.x ? nlong : gridDim.x;
+  const uint32_t nstatic = (gridDim.x - taken) * 2u;   // wavefronts that start on the general queries
+  bool firstQuery = blockIdx.x >= taken;
   for (;;) {
     uint32_t qi = 0;
-    if (lane == 0) qi = atomicAdd(head, 1u);
-    qi = (uint32_t)uniform_i((int)qi);
+    if (firstQuery) {
+      qi = taken + (blockIdx.x - taken) * 2u + (uint32_t)half;
+      firstQuery = false;
+    } else {
+      if (lane == 0) qi = atomicAdd(head, 1u);
+      qi = taken + nstatic + (uint32_t)uniform_i((int)qi);
+    }
     if (qi >= nq) break;
-    if (qi < taken) continue;
     int cls = 0;
     while (qi >= first[cls + 1]) cls++;
     const GeoQuery q = queries[(size_t)cls * stride + (qi - first[cls])];
@@ -674,7 +682,7 @@ __global__ void k_random_points(NavData nav, uint32_t scene, const float* u, uin
 }
 // counts and both ticket counters of a batch of n queries, all in the class of the shortest
 __global__ void k_set_counts(uint32_t* p, uint32_t n) {
-  if (threadIdx.x <= (uint32_t)kGeoClasses + 1u) p[threadIdx.x] = threadIdx.x == (uint32_t)kGeoClasses - 1u ? n : 0u;
+  if (threadIdx.x <= (uint32_t)kGeoClasses) p[threadIdx.x] = threadIdx.x == (uint32_t)kGeoClasses - 1u ? n : 0u;
 }
 
 }  // namespace
@@ -690,9 +698,9 @@ uint32_t geodesic_blocks_per_cu() {
 
 // num_blocks blocks of two wavefronts; slots holds one GeoSlot per wavefront
 void launch_geodesic(const NavData& nav, const GeoQuery* queries, uint32_t stride, const uint32_t* counts, uint32_t* head,
-                     uint32_t* head_long, float* out, uint32_t* last_cost, GeoSlot* slots, uint32_t num_blocks,
+                     float* out, uint32_t* last_cost, GeoSlot* slots, uint32_t num_blocks,
                      uint64_t* counters, hipStream_t st) {
-  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(128), 0, st, nav, queries, stride, counts, head, head_long, out,
+  hipLaunchKernelGGL(k_geodesic, dim3(num_blocks), dim3(128), 0, st, nav, queries, stride, counts, head, out,
                      last_cost, slots, counters);
 }
 
@@ -721,7 +729,7 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   hipLaunchKernelGGL(k_reset_snap, dim3(step_snap_blocks), dim3(128), 0, fork ? side : st, nav, A, Q, Qnext, P);
   if (fork) (void)hipEventRecord(snapped, side);
   mark();
-  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
+  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
   mark();
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
@@ -735,7 +743,7 @@ void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q,
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Qother, Qother);
   hipLaunchKernelGGL(k_reset_all, grid_for(P.n, 256), dim3(256), 0, st, nav, A, Q, P);
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, Q, P);
-  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], &Q.counts[kQGeoHeadLong], A.geo,
+  launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
   hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
   // the next step finds its lists of queries empty, not with this launch's queries still in them
@@ -751,12 +759,12 @@ void launch_try_step_batch(const NavData& nav, uint32_t scene, const float* sxyz
   hipLaunchKernelGGL(k_try_step_batch, grid_for(n, 64), dim3(64), 0, st, nav, scene, sxyz, sref, exyz, n, oxyz, oref);
 }
 void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz, const uint32_t* sref, const float* exyz,
-                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 2] */, float* out,
+                           const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 1] */, float* out,
                            GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st) {
   hipLaunchKernelGGL(k_make_queries, grid_for(n, 256), dim3(256), 0, st, scene, sxyz, sref, exyz, eref, n, qbuf);
   hipLaunchKernelGGL(k_set_counts, dim3(1), dim3(64), 0, st, count_head, n);
   // one class only: stride 0 puts its queries at the start of the buffer
-  launch_geodesic(nav, qbuf, 0, &count_head[0], &count_head[kGeoClasses], &count_head[kGeoClasses + 1], out, nullptr, slots,
+  launch_geodesic(nav, qbuf, 0, &count_head[0], &count_head[kGeoClasses], out, nullptr, slots,
                   geo_blocks, counters, st);
 }
 void launch_set_swap(uint32_t* swap_target, uint32_t* swap_remaining, uint32_t slot, uint32_t target, uint32_t envs,
