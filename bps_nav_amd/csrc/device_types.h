@@ -179,8 +179,14 @@ constexpr uint32_t kNoCostSlot = 0xffffffffu;
 // cost (the nodes the agent's previous searches expanded) and served from the longest class
 // down, which approximates longest-first scheduling; the longer classes also run at a higher
 // issue priority of their wavefront.
-constexpr int kGeoClasses = 16;
-constexpr uint32_t kGeoClassWidth = 100;   // expanded nodes per class: 1500 and more, 1400-1499, ..., below 100
+// The classes are narrow because tickets within a class are served in the order they were
+// queued: the last searches to begin decide when a launch ends, and a class as wide as those
+// searches are long lets one of its longest begin last.
+#ifndef BPSX_GEO_CLASSES
+#define BPSX_GEO_CLASSES 32
+#endif
+constexpr int kGeoClasses = BPSX_GEO_CLASSES;
+constexpr uint32_t kGeoClassWidth = 2048 / BPSX_GEO_CLASSES;   // expanded nodes per class: the last class holds the shortest searches
 constexpr __host__ __device__ uint32_t geo_class(uint32_t last_cost) {
   return last_cost / kGeoClassWidth >= (uint32_t)kGeoClasses ? 0u
                                                              : (uint32_t)kGeoClasses - 1u - last_cost / kGeoClassWidth;

@@ -64,7 +64,7 @@ int dev_alloc(T** p, size_t count) {
 namespace {
 constexpr uint32_t kStaticBlocks = 16;
 constexpr size_t kStaticQueriesBytes = (size_t)BPSX_STATIC_MAX_QUERIES * sizeof(GeoQuery);
-constexpr size_t kStaticCountsBytes = 256;
+constexpr size_t kStaticCountsBytes = 512;
 static_assert((kGeoClasses + 2) * sizeof(uint32_t) <= kStaticCountsBytes, "queue counters must fit their part");
 static_assert(kStaticQueriesBytes % 256 == 0 && sizeof(GeoSlot) % 256 == 0, "parts of the scratch stay aligned");
 constexpr size_t kStaticSlotsBytes = (size_t)kStaticBlocks * 2 * sizeof(GeoSlot);

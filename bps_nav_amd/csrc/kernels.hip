@@ -513,7 +513,7 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
 #endif
   // the longer the expected search, the sooner its instructions issue; a search of unknown
   // length may be among the longest
-  set_wave_priority(cls == (int)kGeoClassUnknown ? 3 : (kGeoClasses - 1 - cls) >> 2);
+  set_wave_priority(cls == (int)kGeoClassUnknown ? 3 : (int)(((uint32_t)(kGeoClasses - 1 - cls) * kGeoClassWidth) / 400u));
 #ifdef BPSX_PHASE_TIMING
   const float d = geodesic_query(g, nav, q, &T.pops, &T.corridor, T.phase_acc);
 #else
@@ -548,7 +548,7 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
 // spills, half the window misses, shorter hash chains; 7 % faster on such searches) while its
 // second wavefront leaves.  Every other wavefront's first query is fixed by its index too;
 // from the second query on a wavefront draws from the queue's counter.
-constexpr int kLongClasses = 2;   // expected cost of 1400 nodes and more
+constexpr int kLongClasses = (int)geo_class(1400);   // the classes of an expected cost of 1400 nodes and more
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) void k_geodesic(NavData nav, const GeoQuery* __restrict__ queries, uint32_t stride,
                                                   const uint32_t* __restrict__ counts, uint32_t* head,
                                                   float* out, uint32_t* last_cost, GeoSlot* slots, uint64_t* counters) {
@@ -557,11 +557,24 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kHalf];
   const int lane = (int)(threadIdx.x & 63), half = uniform_i((int)(threadIdx.x >> 6));   // the same in all lanes, and known to be: addresses derived from it stay in scalar registers
   GeoSlot* slot = &slots[blockIdx.x * 2 + half];
-  // classes are served in order: class c owns ticket numbers [first[c], first[c + 1])
-  uint32_t first[kGeoClasses + 1];
-  first[0] = 0;
-  for (int c = 0; c < kGeoClasses; ++c) first[c + 1] = first[c] + (uint32_t)uniform_i((int)counts[c]);
-  const uint32_t nq = first[kGeoClasses], nlong = first[kLongClasses];
+  // Classes are served in order: class c owns the ticket numbers from the sum of the counts
+  // before it.  A wavefront's tickets only go up, so it keeps the class it is in and that
+  // class's range of tickets, and moves on through the counts as its tickets pass the range.
+  uint32_t nq = 0, nlong = 0;
+  for (int c = 0; c < kGeoClasses; ++c) {
+    nq += (uint32_t)uniform_i((int)counts[c]);
+    if (c + 1 == kLongClasses) nlong = nq;
+  }
+  int curCls = 0;
+  uint32_t curLo = 0, curHi = (uint32_t)uniform_i((int)counts[0]);
+  auto class_of = [&](uint32_t ticket) {   // ticket < nq, not below an earlier one
+    while (ticket >= curHi) {
+      curCls++;
+      curLo = curHi;
+      curHi += (uint32_t)uniform_i((int)counts[curCls]);
+    }
+    return curCls;
+  };
   GeoTotals T;
   uint32_t linkSpills = 0, heapSpills = 0, exactRuns = 0, tieReplays = 0, pairTies = 0;
   // The first query of every wavefront needs no ticket counter: the grid is what the device
@@ -581,9 +594,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
 #ifdef BPSX_TIE_REASONS
     for (int k = 0; k < 8; ++k) gl.why[k] = 0;
 #endif
-    int cls = 0;
-    while (lt >= first[cls + 1]) cls++;
-    const GeoQuery q = queries[(size_t)cls * stride + (lt - first[cls])];
+    const int cls = class_of(lt);
+    const GeoQuery q = queries[(size_t)cls * stride + (lt - curLo)];
     serve_query(gl, nav, q, cls, out, last_cost, T);
     linkSpills += gl.linkSpills; heapSpills += gl.heapSpills; exactRuns += gl.exactRuns; tieReplays += gl.tieReplays; pairTies += gl.pairTies;
     if (lane == 0) atomicAdd((unsigned long long*)&counters[kCntLongPath], 1ull);
@@ -612,9 +624,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
       qi = taken + nstatic + (uint32_t)uniform_i((int)qi);
     }
     if (qi >= nq) break;
-    int cls = 0;
-    while (qi >= first[cls + 1]) cls++;
-    const GeoQuery q = queries[(size_t)cls * stride + (qi - first[cls])];
+    const int cls = class_of(qi);
+    const GeoQuery q = queries[(size_t)cls * stride + (qi - curLo)];
     serve_query(g, nav, q, cls, out, last_cost, T);
   }
   linkSpills += g.linkSpills; heapSpills += g.heapSpills; exactRuns += g.exactRuns; tieReplays += g.tieReplays; pairTies += g.pairTies;
@@ -762,7 +773,7 @@ void launch_geodesic_batch(const NavData& nav, uint32_t scene, const float* sxyz
                            const uint32_t* eref, uint32_t n, GeoQuery* qbuf, uint32_t* count_head /* [kGeoClasses + 1] */, float* out,
                            GeoSlot* slots, uint32_t geo_blocks, uint64_t* counters, hipStream_t st) {
   hipLaunchKernelGGL(k_make_queries, grid_for(n, 256), dim3(256), 0, st, scene, sxyz, sref, exyz, eref, n, qbuf);
-  hipLaunchKernelGGL(k_set_counts, dim3(1), dim3(64), 0, st, count_head, n);
+  hipLaunchKernelGGL(k_set_counts, dim3(1), dim3(128), 0, st, count_head, n);
   // one class only: stride 0 puts its queries at the start of the buffer
   launch_geodesic(nav, qbuf, 0, &count_head[0], &count_head[kGeoClasses], out, nullptr, slots,
                   geo_blocks, counters, st);
