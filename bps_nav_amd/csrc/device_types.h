@@ -191,7 +191,10 @@ constexpr __host__ __device__ uint32_t geo_class(uint32_t last_cost) {
   return last_cost / kGeoClassWidth >= (uint32_t)kGeoClasses ? 0u
                                                              : (uint32_t)kGeoClasses - 1u - last_cost / kGeoClassWidth;
 }
-constexpr uint32_t kGeoClassUnknown = geo_class(700);   // a search without history: upper-middle length
+// A search without history (one in ten) is queued as if it took 1000 nodes: about twice the mean,
+// because one that turns out long and began late is what a launch then waits for, and one that
+// turns out short and began early costs nothing.
+constexpr uint32_t kGeoClassUnknown = geo_class(1000);
 // AgentArrays::last_cost before the episode's first goal -> agent search.  The distance taken at
 // reset is searched the other way round and the previous episode's searches had another goal:
 // neither says how long the first search will be, and it is often among the longest.
