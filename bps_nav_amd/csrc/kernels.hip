@@ -319,7 +319,16 @@ __global__ __launch_bounds__(64) void k_step_move(NavData nav, AgentArrays A, St
   if (i == 0) atomicAdd((unsigned long long*)&P.counters[kCntSteps], (unsigned long long)P.n);
 }
 
-__global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P) {
+// served: the counters of the lists of queries that this step's searches have just served;
+// before: those of the other set.  Both are left as the next step expects them, so that a step
+// needs no launch of its own for it: the served lists and their ticket counter empty, and the
+// reset list of the step before empty (its snaps, which read it, ended before this step began).
+__global__ __launch_bounds__(256) void k_step_finish(AgentArrays A, StepParams P, uint32_t* served, uint32_t* before) {
+  if (blockIdx.x == 0) {
+    static_assert(kQGeoHead == kQGeo + kGeoClasses && kGeoClasses + 1 < 256, "one thread per counter");
+    if (threadIdx.x <= (uint32_t)kGeoClasses) served[kQGeo + threadIdx.x] = 0;
+    else if (threadIdx.x == (uint32_t)kGeoClasses + 1u) before[kQReset] = 0;
+  }
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= P.n) return;
   const uint32_t gi = P.base + i;
@@ -721,9 +730,9 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   int e = 0;
   auto mark = [&]() { if (ev) (void)hipEventRecord(ev[e++], st); };
   mark();
-  // Q's lists of queries were emptied a step ago and have since taken the first queries of the
-  // episodes that began in the previous step; its reset list is emptied now, and so is Qnext
-  hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Qnext, Q);
+  // Q's lists of queries were emptied two steps ago and have since taken the first queries of
+  // the episodes that began in the previous step; its reset list and ticket counter, and the
+  // lists of Qnext, were emptied by the previous step's last launch
   hipLaunchKernelGGL(k_step_move, grid_for(P.n, 64), dim3(64), 0, st, nav, A, Q, P, actions_dev);
   mark();
   // the new episodes' snaps need nothing of this step's searches and the searches nothing of
@@ -743,7 +752,7 @@ void launch_step(const NavData& nav, const AgentArrays& A, const StepQueues& Q, 
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
   mark();
-  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
+  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P, Q.counts, Qnext.counts);
   if (fork) (void)hipStreamWaitEvent(st, snapped, 0);
   mark();
 }
@@ -756,7 +765,7 @@ void launch_reset(const NavData& nav, const AgentArrays& A, const StepQueues& Q,
   hipLaunchKernelGGL(k_reset_snap, dim3(snap_blocks), dim3(128), 0, st, nav, A, Q, Q, P);
   launch_geodesic(nav, Q.queries, Q.stride, &Q.counts[kQGeo], &Q.counts[kQGeoHead], A.geo,
                   A.last_cost, slots, geo_blocks, P.counters, st);
-  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P);
+  hipLaunchKernelGGL(k_step_finish, grid_for(P.n, 256), dim3(256), 0, st, A, P, Q.counts, Qother.counts);
   // the next step finds its lists of queries empty, not with this launch's queries still in them
   hipLaunchKernelGGL(k_clear_queues, dim3(1), dim3(64), 0, st, Q, Q);
 }
