@@ -32,8 +32,7 @@
 // getEdgeMidPoint); DetourNode.cpp:50-200 (node pool, heap order); PathFinder.cpp:473-541.
 //
 // The sizes of the LDS structures are build parameters (BPSX_LINKS_LDS, BPSX_HEAP_LDS,
-// BPSX_WINDOW, BPSX_HASH, BPSX_TAG_SLOTS), as is the number of nodes a pass of the sorted-list
-// loop may expand (BPSX_ROWS: 8 rows of 8 lanes, or 4 of 16), and everything that depends on them lives in namespace
+// BPSX_WINDOW, BPSX_HASH, BPSX_TAG_SLOTS), and everything that depends on them lives in namespace
 // bpsx::BPSX_GEO_NS (default geo): the file can be included again with other values and
 // another namespace name to get a second instantiation of the same search.
 #include "nav_device.h"
@@ -42,18 +41,9 @@
 #define BPSX_GEODESIC_COMMON_H
 namespace bpsx {
 
-#ifdef BPSX_ASM_MARKS
-#define PHASE_MARK(k) asm volatile("; PHASE_MARK " #k)
-#elif defined(BPSX_PHASE_TIMING)
-#define PHASE_MARK(k) do { const unsigned long long now_ = __builtin_readcyclecounter(); phase_acc[k] += now_ - phase_t0; phase_t0 = now_; } while (0)
-#else
-#define PHASE_MARK(k) do { } while (0)
-#endif
-#ifdef BPSX_ASM_MARKS
-#define FM(k) asm volatile("; FAST_MARK " #k)
-#elif defined(BPSX_PHASE_TIMING)
-// marks of the sorted-list loop -> counters: 0 front of the list, 1 fetch, 2 lookup, 3 costs, 4 rows that stand,
-// 5 closing, new nodes and stores, 6 list and log; 7 counts the passes
+#ifdef BPSX_PHASE_TIMING
+// diagnostic build: cycles per phase of the sorted-list loop -> counters: 0 front of the list, 1 fetch, 2 lookup,
+// 3 costs, 4 rows that stand, 5 closing, new nodes and stores, 6 list and log; 7 counts the passes
 #define FM(k) do { constexpr int slot_[11] = {7, 0, 1, 2, 3, 4, 5, 5, 5, 6, 6}; const unsigned long long now_ = __builtin_readcyclecounter(); \
     if ((k) == 0) g.phase[7]++; else g.phase[slot_[k]] += now_ - g.phase_t0; g.phase_t0 = now_; } while (0)
 #else
@@ -203,11 +193,6 @@ struct RegHeap {
     size++;
     bubble_up(size, t, n, lane);
   }
-  // dtNodeQueue::modify: the entry of node n (packed like n0) gets key t and bubbles up
-  BPSX_DEV void modify(uint32_t n, uint32_t t, int lane) {
-    const int q = position(n, lane);
-    if (q) bubble_up(q, t, n, lane);
-  }
   // heap position of node n's entry, 0 if it has none
   template <bool W = true> BPSX_DEV int position(uint32_t n, int lane) const {
     const unsigned long long m0 = lanes_where(lane >= 1 && lane <= size && n0 == n);
@@ -224,14 +209,12 @@ struct RegHeap {
     int q;
     if (open) q = position<W>(n, lane);
     else q = ++size;
-#ifndef BPSX_NO_PUSH_FAST_PATH
     const uint32_t pk = rlane(t0, q >> 1);   // position 0 holds kEmpty: no entry (q = 0) and the root take the walk
     if (pk <= t) {
       if (!W || q < 64) { t0 = wlane(t0, t, q); n0 = wlane(n0, n, q); }
       else { t1 = wlane(t1, t, q & 63); n1 = wlane(n1, n, q & 63); }
       return;
     }
-#endif
     bubble_up<W>(q, t, n, lane);
   }
   // dtNodeQueue::pop after the caller has taken the root.  The reference moves the hole left
@@ -505,13 +488,10 @@ constexpr int kHashSize = BPSX_HASH;        // buckets of the node pool's hash t
 #define BPSX_TAG_SLOTS 256
 #endif
 constexpr int kTagSlots = BPSX_TAG_SLOTS;
-#ifndef BPSX_ROWS
-#define BPSX_ROWS 8
-#endif
-constexpr int kRows = BPSX_ROWS;            // nodes expanded per pass of astar_fast, one per row of 64 / kRows lanes
+constexpr int kRows = 8;                    // nodes expanded per pass of astar_fast, one per row of 64 / kRows lanes
 constexpr int kRowLanes = 64 / kRows;
-constexpr int kRowShift = kRows == 8 ? 3 : 4;
-static_assert((kRows == 4 || kRows == 8) && kRowLanes > kNvp, "a row needs a lane per edge and one for the node itself");
+constexpr int kRowShift = 3;
+static_assert(kRowLanes == (1 << kRowShift) && kRowLanes > kNvp, "a row needs a lane per edge and one for the node itself");
 // lanes of the rows below j
 constexpr unsigned long long rows_below(int j) { return j * kRowLanes >= 64 ? ~0ull : (1ull << (j * kRowLanes)) - 1ull; }
 static_assert((kWindow & (kWindow - 1)) == 0 && kWindow >= 2 * kNvp, "window must be a power of two");
@@ -559,15 +539,6 @@ struct GeoWave {
   uint32_t exactRuns;                // queries run again with the exact heap
   uint32_t tieReplays;               // ties resolved by replaying the operation log through the exact heap
   uint32_t pairTies;                 // passes that took two nodes of equal total in one go
-#ifdef BPSX_TIE_REASONS
-  uint32_t why[8];
-#define TIE_WHY(k) g.why[k]++
-#else
-#define TIE_WHY(k) do { } while (0)
-#endif
-#ifdef BPSX_QUERY_TRACE
-  uint32_t missTop, missNb, maxHeap;
-#endif
 
   // ---------------------------------------------------------------- node pool
   template <bool S> BPSX_DEV uint32_t link(int i) const {
@@ -693,40 +664,21 @@ struct GeoWave {
   }
 };
 
-// The expansion loop of findPath.  M = 0: open list in registers, all links in LDS; M = 1: open
-// list in registers, links may spill; M = 2: open list in LDS/HBM, links may spill.  Returns
-// kAstarGrow* before an expansion that could outgrow what its mode holds.
-template <int M>
-BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
-#ifdef BPSX_PHASE_TIMING
-                              , unsigned long long* phase_acc, unsigned long long& phase_t0
-#endif
-                              ) {
+// The expansion loop of findPath for an open list that has left the registers (more than
+// kRegHeap entries: an obstacle-free hall does it, the benchmark's mazes and rooms do not): the
+// reference's heap in LDS/HBM, one node per pass, links wherever they are.
+BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops) {
   const int lane = g.lane;
   GeoLds* L = g.L;
   const float H_SCALE = 0.999f;
   const float e0 = endPos[0], e1 = endPos[1], e2 = endPos[2];
   endIp = (uint32_t)uniform_i((int)endIp);   // the same in all lanes: the goal test stays on the scalar unit
-  constexpr bool S = M >= 1;    // links and states may be in HBM
-  constexpr bool SH = M == 2;   // open list in LDS/HBM
-  RegHeap& rh = st.rh;
-  while ((SH ? g.heapSize : rh.size) > 0) {
-    if (M == 0 && g.nodeCount > kLinksLds - kNvp) return kAstarGrowLinks;
-    if (!SH && rh.size > kRegHeap - kNvp) return kAstarGrowHeap;
+  constexpr bool S = true;    // links and states may be in HBM
+  while (g.heapSize > 0) {
     // the node about to be popped is the root: fetch its edges while the heap is repaired
-    int bi;
-    uint32_t bestIp;
-    uint32_t blink;   // the node's link word: closing the node rewrites its flags
-    if (SH) {
-      bi = uniform_i((int)L->heap[0].node);
-      blink = g.link<S>(bi);
-      bestIp = link_id((uint32_t)uniform_i((int)blink));
-    } else {
-      const uint32_t root = rlane(rh.n0, 1);
-      bi = (int)(root & 0x7ffu);
-      bestIp = root >> 11;
-      blink = g.link<S>(bi);
-    }
+    const int bi = uniform_i((int)L->heap[0].node);
+    const uint32_t blink = g.link<S>(bi);   // the node's link word: closing the node rewrites its flags
+    const uint32_t bestIp = link_id((uint32_t)uniform_i((int)blink));
     uint32_t nb = kNoNb;
     float m0 = 0, m1 = 0, m2 = 0;
     if (lane < kNvp) {
@@ -738,53 +690,37 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (g.in_window(bi)) {
       const int w = bi & (kWindow - 1);
       b0 = L->w_pos[0][w]; b1 = L->w_pos[1][w]; b2 = L->w_pos[2][w]; bcost = L->w_cost[w];
-      if (!SH) bparent = L->w_parent[w];
-      else { BPSX_KEEP_APART(); bparent = g.ws->nodes[bi].parent; BPSX_KEEP_APART(); }
+      BPSX_KEEP_APART(); bparent = g.ws->nodes[bi].parent; BPSX_KEEP_APART();   // the heap lies over the window's parent indices
     } else {
       BPSX_KEEP_APART();
       const float4 pc = *reinterpret_cast<const float4*>(g.ws->nodes[bi].pos);   // pos, cost
       b0 = pc.x; b1 = pc.y; b2 = pc.z; bcost = pc.w;
       bparent = g.ws->nodes[bi].parent;
       BPSX_KEEP_APART();
-#ifdef BPSX_QUERY_TRACE
-      g.missTop++;
-#endif
     }
-#ifdef BPSX_QUERY_TRACE
-    if (!SH && (uint32_t)rh.size > g.maxHeap) g.maxHeap = (uint32_t)rh.size;
-#endif
-    PHASE_MARK(0);
-    if (SH) g.pop<true>();
-    else rh.pop(lane);
+    g.pop<S>();
     const uint32_t pidx = (uint32_t)uniform_i((int)bparent);
-    PHASE_MARK(1);
     g.set_link<S>(bi, with_flags(blink, 2u));   // open -> closed
     if (bestIp == endIp) { st.lastBest = bi; return kAstarGoal; }
     (*pops)++;
-    PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
     uint32_t chainHead, hitLink;
     int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
     // the polygon the expanded node was reached from is not entered again
     if (pidx && ni + 1 == (int)pidx) nb = kNoNb;
-    PHASE_MARK(3);
-    // new nodes take consecutive indices in edge order; past the pool's end they are dropped
+    // new nodes take consecutive indices in edge order
     const bool isNew = nb != kNoNb && ni < 0;
     const unsigned long long need = lanes_where(isNew);
     if (need) {
       const int rank = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(need >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)need, 0u));
       const int count = __popcll(need);
-      if (isNew) {
-        const int idx = g.nodeCount + rank;
-        if (!S || idx < kMaxNodes) ni = idx;
-        else nb = kNoNb;
-      }
       const int want = g.nodeCount + count;
-      // the reference carries on without the dropped nodes, but reports anything found after
-      // that as failure (only plain DT_SUCCESS counts, PathFinder.cpp:506): the search can stop
-      if (S && want > kMaxNodes) { st.outOfNodes = true; return kAstarEmpty; }
-      g.nodeCount = (!S || want < kMaxNodes) ? want : kMaxNodes;
-      bool pending = isNew && nb != kNoNb;
+      // the reference carries on without the nodes that do not fit, but reports anything found
+      // after that as failure (only plain DT_SUCCESS counts, PathFinder.cpp:506): the search can stop
+      if (want > kMaxNodes) { st.outOfNodes = true; return kAstarEmpty; }
+      if (isNew) ni = g.nodeCount + rank;
+      g.nodeCount = want;
+      bool pending = isNew;
       // All insert at once in front of the chain head their lookup saw.  Of several that share a
       // bucket one store wins; the others see that when they read the head back and go round
       // again behind the winner.  One new node needs no check.  A new node is open from the
@@ -805,10 +741,6 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
         if (!lanes_where(pending)) break;
       }
     }
-    PHASE_MARK(4);
-#ifdef BPSX_QUERY_TRACE
-    g.missNb += (uint32_t)__popcll(lanes_where(nb != kNoNb && !isNew && !g.in_window(ni)));
-#endif
     // Costs of the step to each neighbour (lane-wise).  Written with few branches: all lanes
     // issue the one round of LDS reads a revisited node needs (idle lanes read slot 0; its flags
     // came with the lookup), the rare node that has left the window is fetched under a
@@ -849,35 +781,25 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
       if (inw) {
         L->w_pos[0][w] = p0; L->w_pos[1][w] = p1; L->w_pos[2][w] = p2;   // unchanged for a revisited node
         L->w_cost[w] = cost; L->w_total[w] = total;
-        if (!SH) L->w_parent[w] = (uint16_t)(bi + 1);
       }
       *reinterpret_cast<float4*>(hn.pos) = make_float4(p0, p1, p2, cost);
       *reinterpret_cast<uint2*>(&hn.total) = make_uint2(__float_as_uint(total), (uint32_t)(bi + 1));   // total, parent = expanded node
       g.ws->parents[ni] = (uint16_t)(bi + 1);
     }
     wave_sync();
-    PHASE_MARK(5);
     // ---- ordered phase, in edge order: the open list.  (findPath's "nearest so far" record,
     // lastBestNode, is not kept: it only matters to a search that ends without reaching the
     // goal, and the caller reports DT_PARTIAL_RESULT as failure, PathFinder.cpp:506.)
-    const uint32_t packed = (uint32_t)ni | (nb << 11);   // heap entry of this lane's node
     unsigned long long upd = lanes_where(update);
     const unsigned long long openMask = lanes_where(wasOpen);
     while (upd) {
       const int src = __ffsll((long long)upd) - 1;
       upd &= upd - 1;
-      const uint32_t entry = rlane(packed, src);
+      const int node = (int)rlane((uint32_t)ni, src);
       const float t = lane_f(total, src);
-      const bool open = (openMask >> src) & 1ull;
-      if (SH) {
-        if (open) g.modify<true>((int)(entry & 0x7ffu), t);
-        else g.push<true>(t, (int)(entry & 0x7ffu));
-      } else {
-        if (open) rh.modify(entry, __float_as_uint(t), lane);
-        else rh.push(__float_as_uint(t), entry, lane);
-      }
+      if ((openMask >> src) & 1ull) g.modify<S>(node, t);
+      else g.push<S>(t, node);
     }
-    PHASE_MARK(6);
   }
   return kAstarEmpty;
 }
@@ -897,11 +819,7 @@ BPSX_DEV AstarExit astar_loop(GeoWave& g, AstarState& st, const AEdge* edges, ui
 // list see A's updates in edge order, then B's pop, then B's updates.  Otherwise B's lanes
 // are dropped and B becomes A of the next pass.
 template <bool S, bool W>
-BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops
-#ifdef BPSX_PHASE_TIMING
-                               , unsigned long long* phase_acc, unsigned long long& phase_t0
-#endif
-                               ) {
+BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, uint32_t endIp, const float* endPos, uint32_t* pops) {
   const int lane = g.lane;
   GeoLds* L = g.L;
   const float H_SCALE = 0.999f;
@@ -951,19 +869,15 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
         }
       }
     }
-    PHASE_MARK(0);
     rh.template pop<W>(lane);
-    PHASE_MARK(1);
     g.set_link<S>(biA, with_flags(blinkA, 2u));   // open -> closed
     if (ipA == endIp) { st.lastBest = biA; return kAstarGoal; }
     (*pops)++;
-    PHASE_MARK(2);
     const uint32_t bucket = GeoWave::hash(nb);
     uint32_t chainHead, hitLink;
     int ni = g.find<S>(nb != kNoNb, nb, bucket, &chainHead, &hitLink);
     // the polygon the expanded node was reached from is not entered again
     if (bparent && ni + 1 == (int)bparent) nb = kNoNb;
-    PHASE_MARK(3);
     // ---- costs of both nodes' steps (new nodes have no index yet and read slot 0)
     const bool isNew = nb != kNoNb && ni < 0;
     const bool valid = nb != kNoNb;
@@ -1005,7 +919,6 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
     }
     update = update & (!rowB | two);   // B's lanes are dropped unless B stands
     const bool wasOpen = update && (fl & 1u) != 0;
-    PHASE_MARK(4);
     // ---- new nodes take consecutive indices in edge order, A's before B's
     {
       const bool mine = isNew && update;   // a new node is always taken
@@ -1055,7 +968,6 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       g.ws->parents[ni] = (uint16_t)parent;
     }
     wave_sync();
-    PHASE_MARK(5);
     // ---- ordered phase, in the reference's order: A's lanes come before B's.  (findPath's
     // "nearest so far" record, lastBestNode, is not kept: it only matters to a search that ends
     // without reaching the goal, which the caller reports as failure, PathFinder.cpp:506.)
@@ -1074,12 +986,8 @@ BPSX_DEV AstarExit astar_loop2(GeoWave& g, AstarState& st, const AEdge* edges, u
       rh.template pop<W>(lane);
       g.set_link<S>(biB, with_flags(blinkB, 2u));
       (*pops)++;
-#ifdef BPSX_PHASE_TIMING
-      phase_acc[7]++;   // passes that expanded two nodes
-#endif
       apply(upd & ~0xffffull);
     }
-    PHASE_MARK(6);
   }
   return kAstarEmpty;
 }
@@ -1118,7 +1026,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
   const int row = lane >> kRowShift, el = lane & (kRowLanes - 1);
   const bool edgeLane = el < kNvp;
   const bool ownLane = el == kNvp;   // looks after the row's own node in the conflict test
-  constexpr unsigned long long kRowStart = kRows == 8 ? 0x0101010101010101ull : 0x0001000100010001ull;
+  constexpr unsigned long long kRowStart = 0x0101010101010101ull;   // the first lane of every row
   constexpr unsigned long long kRows1 = rows_below(1), kRows2 = rows_below(2);   // lanes of the first rows
   unsigned long long resolved = frontResolved ? 1ull : 0ull;
   // Written for few instructions on the common path: what is rare sits behind one branch each,
@@ -1129,7 +1037,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     if (!S && g.nodeCount > kLinksLds - kRows * kNvp) return kAstarGrowLinks;
     if (st.logEnd > kOpLogCap - (1 + kRows * kNvp)) return kAstarLogFull;
     FM(0);
-    TIE_WHY(7);   // passes
     // ---- how many entries at the front are each the only one with their total
     const unsigned long long uniq = lanes_where(ol.t[0] < OpenList::down1(OpenList::kEmpty, ol.t[0]));
     int lim = __builtin_ctzll(~uniq | (1ull << kRows));
@@ -1147,7 +1054,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         // whatever they put on the list lies above their total), the reference expands them one
         // after the other, in the order its heap has them in, and ends in the same state either
         // way: the pass takes both and notes in the log that their order is open.
-        if (!(uniq & 2ull)) { TIE_WHY(0); return kAstarTie; }
+        if (!(uniq & 2ull)) return kAstarTie;
         pairTie = true;
         g.pairTies++;   // counts the attempts: one that fails comes back through the log
         rowsAt1 = kRows2;
@@ -1215,15 +1122,8 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const float ex = e0 - p0, ey = e1 - p1, ez = e2 - p2;
     const float cc = cx * cx + cy * cy + cz * cz, ee = ex * ex + ey * ey + ez * ez;
     float curCost, toEnd;
-    if (kRowLanes == 16) {
-      // both roots in one evaluation: the upper half of a row is idle
-      const float roots = sqrt_exact(lanes_up8(cc, ee));
-      curCost = roots * 1.0f;
-      toEnd = lanes_down8(roots);
-    } else {
-      sqrt_exact2(cc, ee, &curCost, &toEnd);
-      curCost = curCost * 1.0f;
-    }
+    sqrt_exact2(cc, ee, &curCost, &toEnd);
+    curCost = curCost * 1.0f;
     const bool last = nb == endIp;
     const float cost = last ? bcost + curCost + toEnd * 1.0f : bcost + curCost;
     const float heuristic = last ? 0.0f : toEnd * H_SCALE;
@@ -1239,7 +1139,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       // holds them (an exhausted pool is reported as failure).  Otherwise the heap must say.
       const unsigned long long touches = lanes_where(tb != 0xffffffffu && ni >= 0);
       const int fresh = __popcll(lanes_where(tb != 0xffffffffu));
-      if (touches || g.nodeCount + fresh > kMaxNodes) { TIE_WHY(1); return kAstarTie; }
+      if (touches || g.nodeCount + fresh > kMaxNodes) return kAstarTie;
       const int biG = (int)rlane((uint32_t)bi, first_lane(goal & kRows2));
       g.set_link<S>(biG, with_flags(g.link<S>(biG), 2u));
       st.lastBest = biG;
@@ -1274,7 +1174,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
       // rows 0 and 1 of a tied pair in either order: row 0 must not read what row 1 updates either
       if (__builtin_expect(pairTie, 0)) {
         pairFails = c < 2 || (lanes_where(seenr == 1u) & kRows1) != 0;
-        if (pairFails && jv < 2) TIE_WHY(2);
         if (pairFails && jv >= 2) {
           // The marks are kept per polygon hash, and a pair that fails costs a replay of the log:
           // the polygons that either row updates are compared with those the other row reads,
@@ -1288,7 +1187,7 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
             const unsigned long long others = src < kRowLanes ? (kRows2 & ~kRows1) : kRows1;
             if (lanes_where(readPoly == rlane(nb, src)) & others) real = true;
           }
-          if (!real) { pairFails = false; c = 2; TIE_WHY(4); } else TIE_WHY(3);
+          if (!real) { pairFails = false; c = 2; }
         }
       }
     }
@@ -1385,15 +1284,8 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
 // Runs A* for one query. Returns the corridor length (corridor written to F->corridor), or 0
 // when the reference would report anything but plain DT_SUCCESS.
 BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev& s, uint32_t startIp, uint32_t endIp,
-                   const float* startPos, const float* endPos, uint32_t* pops
-#ifdef BPSX_PHASE_TIMING
-                   , unsigned long long* phase_acc
-#endif
-                   ) {
+                   const float* startPos, const float* endPos, uint32_t* pops) {
   const int lane = g.lane;
-#ifdef BPSX_PHASE_TIMING
-  unsigned long long phase_t0 = __builtin_readcyclecounter();
-#endif
   if (startIp == endIp) {
     if (lane == 0) F->corridor[0] = (uint16_t)startIp;
     wave_sync();
@@ -1401,19 +1293,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
   }
   AstarState st;
   const AEdge* edges = nav.aedges + (size_t)(uint32_t)uniform_i((int)s.poly_base) * kEdgeStride;
-#ifdef BPSX_PHASE_TIMING
-#define ASTAR_ARGS g, st, edges, endIp, endPos, pops, phase_acc, phase_t0
-#else
 #define ASTAR_ARGS g, st, edges, endIp, endPos, pops
-#endif
-#define ASTAR_RUN(M) astar_loop<M>(ASTAR_ARGS)
   const uint32_t pops0 = *pops;
   AstarExit ex;
-#ifdef BPSX_EXACT_ONLY
-  bool exact = true;
-#else
-  bool exact = false;   // first with the sorted open list; with the reference's heap when that meets a tie
-#endif
+  bool exact = false;   // first with the sorted open list; with the exact loops when that cannot go on
   for (;;) {
     g.clear();
     const float dx = endPos[0] - startPos[0], dy = endPos[1] - startPos[1], dz = endPos[2] - startPos[2];
@@ -1439,7 +1322,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
     bool spill = false, wide = false;
     if (!exact) {
 #ifdef BPSX_PHASE_TIMING
-      for (int k = 0; k < 8; ++k) g.phase[k] = 0;
       g.phase_t0 = __builtin_readcyclecounter();
 #endif
       st.ol.init();
@@ -1471,14 +1353,8 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         __builtin_amdgcn_s_setprio(3);   // a search that pays for a replay is late from here on
         // a tie: the reference pops what its heap has at the root, so the heap is brought up to
         // date from the log, and that entry goes first
-#ifdef BPSX_TIE_REASONS
-        g.why[6] += (uint32_t)(st.logEnd - st.synced);   // records that the replay goes through
-#endif
         if (!replay_log(g.ws->oplog, st, lane) || st.rh.size != st.ol.size) { restart = true; break; }
         g.tieReplays++;
-#ifdef BPSX_TIE_REASONS
-        g.why[5] += *pops - pops0;   // nodes expanded so far when the log is replayed
-#endif
         const uint32_t root = rlane(st.rh.n0, 1);
         const unsigned long long at = lanes_where(st.ol.n[0] == root);
         const int p = at ? __ffsll((long long)at) - 1 : -1;
@@ -1488,10 +1364,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         st.ol.n[0] = wlane(st.ol.n[0], front, p);
         resolved = true;
       }
-#ifdef BPSX_PHASE_TIMING
-      for (int k = 0; k < 8; ++k) phase_acc[k] += g.phase[k];
-      phase_t0 = __builtin_readcyclecounter();
-#endif
       if (restart) {
         g.exactRuns++;
         *pops = pops0;
@@ -1500,10 +1372,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       }
       break;
     }
-#ifdef BPSX_ONE_NODE_PER_PASS
-    ex = ASTAR_RUN(0);
-    if (ex == kAstarGrowLinks) { g.linkSpills++; ex = ASTAR_RUN(1); }
-#else
     {
       wide = false;
       for (;;) {
@@ -1514,7 +1382,6 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
         else break;
       }
     }
-#endif
     if (ex == kAstarGrowHeap) {
       g.heapSpills++;
       // the open list leaves the registers: entry q goes to index q - 1 of the LDS heap
@@ -1528,11 +1395,10 @@ BPSX_DEV int astar(GeoWave& g, FunnelLds* F, const NavData& nav, const SceneDev&
       if (64 + lane <= rh.size) put(63 + lane, rh.t1, rh.n1);
       g.heapSize = rh.size;
       wave_sync();
-      ex = ASTAR_RUN(2);
+      ex = astar_loop(ASTAR_ARGS);
     }
     break;
   }
-#undef ASTAR_RUN
 #undef ASTAR_ARGS
   // an open list that ran empty, or a pool that ran out, is DT_PARTIAL_RESULT or
   // DT_OUT_OF_NODES in the reference: no path to build, the result is a failure
@@ -1671,11 +1537,7 @@ BPSX_DEV float funnel_length(int lane, FunnelLds* F, const NavData& nav, const S
 }
 
 // Full PathFinder::findPath distance for one query, executed by a wavefront.
-BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q, uint32_t* pops, uint32_t* corridor
-#ifdef BPSX_PHASE_TIMING
-                              , unsigned long long* phase_acc
-#endif
-                              ) {
+BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q, uint32_t* pops, uint32_t* corridor) {
   const float INF = __int_as_float(0x7f800000);
   {
     // Eigen isApprox with default precision; sums of three reduce as a0 + (a1 + a2)
@@ -1693,16 +1555,10 @@ BPSX_DEV float geodesic_query(GeoWave& g, const NavData& nav, const GeoQuery& q,
   if (nav.polys[s.poly_base + sIp].island != nav.polys[s.poly_base + eIp].island) return INF;
   if (!finite3(q.a[0], q.a[1], q.a[2]) || !finite3(q.b[0], q.b[1], q.b[2])) return INF;
   FunnelLds* F = &reinterpret_cast<GeoShared*>(g.L)->f;
-#ifdef BPSX_PHASE_TIMING
-  const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops, phase_acc);
-  unsigned long long phase_t0 = __builtin_readcyclecounter();
-#else
   const int n = astar(g, F, nav, s, sIp, eIp, q.a, q.b, pops);
-#endif
   if (n <= 0) return INF;
   *corridor += (uint32_t)n;
   const float len = funnel_length(g.lane, F, nav, s, n, q.a, q.b);
-  PHASE_MARK(7);
   return len;
 }
 

@@ -40,10 +40,7 @@
 #define BPSX_LINKS_LDS 2048
 #define BPSX_HEAP_LDS 32
 #define BPSX_WINDOW 256
-#ifndef BPSX_LONG_HASH
-#define BPSX_LONG_HASH 1024
-#endif
-#define BPSX_HASH BPSX_LONG_HASH
+#define BPSX_HASH 1024
 #include "geodesic_device.h"
 #include "kernels.h"
 
@@ -507,27 +504,19 @@ __global__ __launch_bounds__(128) void k_reset_snap(NavData nav, AgentArrays A, 
 // result and the agent's cost estimate.
 struct GeoTotals {
   uint32_t pops = 0, corridor = 0, done = 0;
-#ifdef BPSX_PHASE_TIMING
-  unsigned long long phase_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
 };
 template <class Wave>
 BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cls, float* out, uint32_t* last_cost, GeoTotals& T) {
   const uint32_t pops0 = T.pops;
 #ifdef BPSX_QUERY_TRACE
   const unsigned long long trace_t0 = wall_clock64();
-  g.missTop = g.missNb = g.maxHeap = 0;
   const uint32_t trace_replays0 = g.tieReplays, trace_spills0 = g.linkSpills, trace_bridges0 = g.exactRuns;
   const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
   // the longer the expected search, the sooner its instructions issue; a search of unknown
   // length may be among the longest
   set_wave_priority(cls == (int)kGeoClassUnknown ? 3 : (int)(((uint32_t)(kGeoClasses - 1 - cls) * kGeoClassWidth) / 400u));
-#ifdef BPSX_PHASE_TIMING
-  const float d = geodesic_query(g, nav, q, &T.pops, &T.corridor, T.phase_acc);
-#else
   const float d = geodesic_query(g, nav, q, &T.pops, &T.corridor);
-#endif
   if (g.lane == 0) {
 #ifdef BPSX_QUERY_TRACE
     const unsigned int ti = atomicAdd(&g_trace_n, 1u);
@@ -600,14 +589,17 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     gl.heapSize = 0;
     gl.nodeCount = 0;
     gl.linkSpills = gl.heapSpills = gl.exactRuns = gl.tieReplays = gl.pairTies = 0;
-#ifdef BPSX_TIE_REASONS
-    for (int k = 0; k < 8; ++k) gl.why[k] = 0;
+#ifdef BPSX_PHASE_TIMING
+    for (int k = 0; k < 8; ++k) gl.phase[k] = 0;
 #endif
     const int cls = class_of(lt);
     const GeoQuery q = queries[(size_t)cls * stride + (lt - curLo)];
     serve_query(gl, nav, q, cls, out, last_cost, T);
     linkSpills += gl.linkSpills; heapSpills += gl.heapSpills; exactRuns += gl.exactRuns; tieReplays += gl.tieReplays; pairTies += gl.pairTies;
     if (lane == 0) atomicAdd((unsigned long long*)&counters[kCntLongPath], 1ull);
+#ifdef BPSX_PHASE_TIMING
+    if (lane == 0) for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], gl.phase[k]);
+#endif
   }
   geo::GeoWave g;
   g.lane = lane;
@@ -616,8 +608,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
   g.heapSize = 0;
   g.nodeCount = 0;
   g.linkSpills = g.heapSpills = g.exactRuns = g.tieReplays = g.pairTies = 0;
-#ifdef BPSX_TIE_REASONS
-  for (int k = 0; k < 8; ++k) g.why[k] = 0;
+#ifdef BPSX_PHASE_TIMING
+  for (int k = 0; k < 8; ++k) g.phase[k] = 0;
 #endif
   // tickets below `taken` went to the blocks' first wavefronts above
   const uint32_t taken = nlong < gridDim.x ? nlong : gridDim.x;
@@ -647,11 +639,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(5, 5))) voi
     if (exactRuns) atomicAdd((unsigned long long*)&counters[kCntExactRuns], (unsigned long long)exactRuns);
     if (tieReplays) atomicAdd((unsigned long long*)&counters[kCntTieReplays], (unsigned long long)tieReplays);
     if (pairTies) atomicAdd((unsigned long long*)&counters[kCntPairTies], (unsigned long long)pairTies);
-#ifdef BPSX_TIE_REASONS
-    for (int k = 0; k < 8; ++k) if (g.why[k]) atomicAdd((unsigned long long*)&counters[8 + k], (unsigned long long)g.why[k]);
-#endif
 #ifdef BPSX_PHASE_TIMING
-    for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], T.phase_acc[k]);
+    for (int k = 0; k < 8; ++k) atomicAdd((unsigned long long*)&counters[8 + k], g.phase[k]);
 #endif
   }
 }

@@ -24,6 +24,13 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* The library is built with hidden visibility: the functions declared here, and nothing else,
+ * are exported. */
+#if defined(__GNUC__)
+#define BPSX_API __attribute__((visibility("default")))
+#else
+#define BPSX_API
+#endif
 
 #define BPSX_OK 0
 #define BPSX_E_INVAL (-1)    /* bad argument / bad navmesh bytes                    */
@@ -106,7 +113,7 @@ typedef struct bpsx_state {
 } bpsx_state;
 
 /* ---- simulator lifecycle (RolloutGenerator ctor, simulator.cpp:1463-1617) ---- */
-int bpsx_create(const bpsx_config *cfg, bpsx_sim **out);
+BPSX_API int bpsx_create(const bpsx_config *cfg, bpsx_sim **out);
 /* Adds one scene of the dataset: the bytes of a habitat ".navmesh" file (PathFinder::loadNavMesh,
  * PathFinder.cpp:330-408) and its episode table, E rows of 10 floats
  * {start xyz, start rotation xyzw, goal xyz} (struct Episode, simulator.cpp:83-87).
@@ -114,12 +121,12 @@ int bpsx_create(const bpsx_config *cfg, bpsx_sim **out);
  * num_active_scenes scenes must be added; of more, finalize picks the ones that start
  * resident at random (Dataset + the selection loop of simulator.cpp:1518-1534, on the
  * simulator's seed) and, with bpsx_config.rotate_scenes, the others come in over time. */
-int bpsx_add_scene(bpsx_sim *sim, const void *navmesh_bytes, size_t navmesh_size,
+BPSX_API int bpsx_add_scene(bpsx_sim *sim, const void *navmesh_bytes, size_t navmesh_size,
                    const float *episodes, uint32_t num_episodes);
 /* Uploads all scenes, assigns envs to scenes in contiguous blocks of
  * N/num_active_scenes (simulator.cpp:1205-1221) and allocates state. */
-int bpsx_finalize(bpsx_sim *sim);
-void bpsx_destroy(bpsx_sim *sim);
+BPSX_API int bpsx_finalize(bpsx_sim *sim);
+BPSX_API void bpsx_destroy(bpsx_sim *sim);
 
 /* Scene rotation (SceneSwapper / SceneTracker, simulator.cpp:1063-1178, 1284-1310, 1636-1642):
  * swap_scene uploads a new scene for scene slot `slot` (0..num_active_scenes-1).  From then
@@ -130,11 +137,11 @@ void bpsx_destroy(bpsx_sim *sim);
  * returns when it is resident (uploaded on a stream of the library's own).  Must not be
  * called between step_start and step_end.  BPSX_E_UNSUPPORTED if the scene does not fit the
  * space reserved at finalize (bpsx_config.scene_reserve). */
-int bpsx_swap_scene(bpsx_sim *sim, uint32_t slot, const void *navmesh_bytes, size_t navmesh_size,
+BPSX_API int bpsx_swap_scene(bpsx_sim *sim, uint32_t slot, const void *navmesh_bytes, size_t navmesh_size,
                     const float *episodes, uint32_t num_episodes);
 /* Envs of the slot that are still on the old scene (0: no swap in progress), and the number
  * of swaps completed over all slots since creation (swap_stats, simulator.cpp:1412-1424). */
-int bpsx_swap_status(bpsx_sim *sim, uint32_t slot, uint32_t *envs_remaining, uint64_t *swaps_completed);
+BPSX_API int bpsx_swap_status(bpsx_sim *sim, uint32_t slot, uint32_t *envs_remaining, uint64_t *swaps_completed);
 
 /* Automatic rotation (bpsx_config.rotate_scenes): a loader thread inside the library parses and
  * uploads the next scene of a slot on a stream of its own while the simulation steps;
@@ -148,14 +155,14 @@ int bpsx_swap_status(bpsx_sim *sim, uint32_t slot, uint32_t *envs_remaining, uin
  * its own simulator); also returns BPSX_E_INVAL once if the loader thread failed on a scene.
  * swap_stats: {swaps completed per 100 env steps, scenes in use, envs per scene} as the
  * reference's swap_stats property computes them (simulator.cpp:1412-1424). */
-int bpsx_active_scenes(bpsx_sim *sim, uint32_t *out /* [num_active_scenes] */);
-int bpsx_rotation_log(bpsx_sim *sim, uint32_t *out /* [max_rows][3] */, uint32_t max_rows, uint32_t *num_rows);
-int bpsx_swap_stats(bpsx_sim *sim, double *out /* [3] */);
+BPSX_API int bpsx_active_scenes(bpsx_sim *sim, uint32_t *out /* [num_active_scenes] */);
+BPSX_API int bpsx_rotation_log(bpsx_sim *sim, uint32_t *out /* [max_rows][3] */, uint32_t max_rows, uint32_t *num_rows);
+BPSX_API int bpsx_swap_stats(bpsx_sim *sim, double *out /* [3] */);
 
 /* ---- stepping (simulator.cpp:1377-1410) ---- */
-int bpsx_num_groups(const bpsx_sim *sim, uint32_t *out);
+BPSX_API int bpsx_num_groups(const bpsx_sim *sim, uint32_t *out);
 /* reset(group): every env of the group starts a new episode; only polars is written. */
-int bpsx_reset(bpsx_sim *sim, uint32_t group, void *hip_stream);
+BPSX_API int bpsx_reset(bpsx_sim *sim, uint32_t group, void *hip_stream);
 /* step_start(group, actions): actions int64[n] in {0 stop, 1 forward, 2 left, 3 right};
  * actions_on_device != 0 => device pointer (read in stream order), else host pointer
  * (copied before returning).  Enqueues the step; returns without waiting.  Part of the step
@@ -164,14 +171,14 @@ int bpsx_reset(bpsx_sim *sim, uint32_t group, void *hip_stream);
  * whole step.  The first distance of an episode that begins in a step is measured by the next
  * step (the reference measures it at once, simulator.cpp:744-751, and uses it from the next
  * step on): outputs and state arrays are the same after every step. */
-int bpsx_step_start(bpsx_sim *sim, uint32_t group, const int64_t *actions,
+BPSX_API int bpsx_step_start(bpsx_sim *sim, uint32_t group, const int64_t *actions,
                     int actions_on_device, void *hip_stream);
 /* step_end(group): waits until the step's outputs are complete. */
-int bpsx_step_end(bpsx_sim *sim, uint32_t group);
-int bpsx_get_outputs(bpsx_sim *sim, uint32_t group, bpsx_outputs *out);
-int bpsx_get_state(bpsx_sim *sim, uint32_t group, bpsx_state *out);
+BPSX_API int bpsx_step_end(bpsx_sim *sim, uint32_t group);
+BPSX_API int bpsx_get_outputs(bpsx_sim *sim, uint32_t group, bpsx_outputs *out);
+BPSX_API int bpsx_get_state(bpsx_sim *sim, uint32_t group, bpsx_state *out);
 /* Sticky error flag raised by kernels (invalid action ids): 0 or BPSX_E_ACTION. */
-int bpsx_check_errors(bpsx_sim *sim);
+BPSX_API int bpsx_check_errors(bpsx_sim *sim);
 /* Counters accumulated by the kernels since creation (u64 each):
  * [0] agent-steps, [1] forward moves, [2] geodesic queries, [3] A* nodes expanded,
  * [4] corridor polygons string-pulled, [5] resets, [6] polygons visited by moves,
@@ -189,30 +196,30 @@ int bpsx_check_errors(bpsx_sim *sim);
  * sorted form's 256 entries or the heap outgrew the registers during a rebuild.  Same results in
  * all cases. */
 #define BPSX_NUM_COUNTERS 22
-int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
+BPSX_API int bpsx_get_counters(bpsx_sim *sim, uint64_t *out /* [BPSX_NUM_COUNTERS] */);
 /* Per-kernel timing with HIP events on the step's own stream. While enabled, every
  * step records a timestamp before each of its BPSX_NUM_KERNELS launches; step_end adds the
  * elapsed times up.  get_kernel_times returns the sums in milliseconds and the number of
  * steps they cover; enabling clears the sums. */
 #define BPSX_NUM_KERNELS 4
-int bpsx_set_profiling(bpsx_sim *sim, int enabled);
-int bpsx_get_kernel_times(bpsx_sim *sim, double *out_ms_sum /* [BPSX_NUM_KERNELS] */,
+BPSX_API int bpsx_set_profiling(bpsx_sim *sim, int enabled);
+BPSX_API int bpsx_get_kernel_times(bpsx_sim *sim, double *out_ms_sum /* [BPSX_NUM_KERNELS] */,
                           uint64_t *out_steps);
-const char *bpsx_kernel_name(uint32_t idx);
+BPSX_API const char *bpsx_kernel_name(uint32_t idx);
 
 /* ---- batched PathFinder queries on one uploaded scene (PathFinder.h:99-227) ----
  * All pointers are host pointers; n items; results copied back before returning. */
 /* snapPoint (PathFinder.cpp:573-584): pts f32[n][3] -> out_xyz f32[n][3] (NaN on failure),
  * out_ref u32[n] (0 on failure). */
-int bpsx_snap_points(bpsx_sim *sim, uint32_t scene, const float *pts, uint32_t n,
+BPSX_API int bpsx_snap_points(bpsx_sim *sim, uint32_t scene, const float *pts, uint32_t n,
                      float *out_xyz, uint32_t *out_ref);
 /* tryStep with sliding (PathFinder.cpp:543-571). */
-int bpsx_try_steps(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
+BPSX_API int bpsx_try_steps(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
                    const uint32_t *start_ref, const float *end_xyz, uint32_t n,
                    float *out_xyz, uint32_t *out_ref);
 /* findPath geodesic distance (PathFinder.cpp:485-541): +inf when unreachable or when a
  * Detour buffer limit is hit, 0 for coincident points. */
-int bpsx_geodesic(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
+BPSX_API int bpsx_geodesic(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
                   const uint32_t *start_ref, const float *end_xyz, const uint32_t *end_ref,
                   uint32_t n, float *out_dist);
 /* bpsx_geodesic for callers that cannot allocate (code under HIP graph capture, tight serving
@@ -225,16 +232,16 @@ int bpsx_geodesic(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
  * that array: calls that overlap on one GPU (other streams, other simulators) race; calls on
  * one stream are safe.  Must not be called between step_start and step_end. */
 #define BPSX_STATIC_MAX_QUERIES 4096
-int bpsx_geodesic_static(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
+BPSX_API int bpsx_geodesic_static(bpsx_sim *sim, uint32_t scene, const float *start_xyz,
                          const uint32_t *start_ref, const float *end_xyz, const uint32_t *end_ref,
                          uint32_t n, float *out_dist, void *hip_stream);
 /* Area-weighted random navigable points (PathFinder.cpp:463-470; distribution of
  * dtNavMeshQuery::findRandomPoint, DetourNavMeshQuery.cpp:220-313).  u f32[n][3] are
  * uniform variates in [0,1): polygon pick, s, t. */
-int bpsx_random_points(bpsx_sim *sim, uint32_t scene, const float *u, uint32_t n,
+BPSX_API int bpsx_random_points(bpsx_sim *sim, uint32_t scene, const float *u, uint32_t n,
                        float *out_xyz, uint32_t *out_ref);
 
-const char *bpsx_last_error(void);
+BPSX_API const char *bpsx_last_error(void);
 
 /* ---- navmesh producer (dtCreateNavMeshData, DetourNavMeshBuilder.cpp:280-658, and the
  * MSET container of PathFinder::saveNavMesh, PathFinder.cpp:410-450) ---- */
@@ -255,12 +262,12 @@ typedef struct bpsx_tile_desc {
   uint32_t build_bv_tree;
 } bpsx_tile_desc;
 /* Builds one Detour tile blob. *out is malloc'd; release with bpsx_free. */
-int bpsx_pack_tile(const bpsx_tile_desc *desc, uint8_t **out, size_t *out_size);
+BPSX_API int bpsx_pack_tile(const bpsx_tile_desc *desc, uint8_t **out, size_t *out_size);
 /* Wraps tile blobs into an MSET ".navmesh" byte string. */
-int bpsx_pack_mset(const uint8_t *const *tiles, const size_t *tile_sizes, uint32_t num_tiles,
+BPSX_API int bpsx_pack_mset(const uint8_t *const *tiles, const size_t *tile_sizes, uint32_t num_tiles,
                    const float orig[3], float tile_width, float tile_height,
                    uint32_t max_tiles, uint32_t max_polys, uint8_t **out, size_t *out_size);
-void bpsx_free(void *p);
+BPSX_API void bpsx_free(void *p);
 
 /* ---- synthetic floor plans (benchmark inputs; no counterpart in the reference, which
  * trains on Gibson/MP3D navmeshes) ---- */
@@ -288,10 +295,10 @@ typedef struct bpsx_scene_params {
   uint32_t tiles_x, tiles_z;     /* split the floor into this many navmesh tiles (0 = 1) */
 } bpsx_scene_params;
 /* Generates one scene as MSET bytes (malloc'd, release with bpsx_free). */
-int bpsx_gen_scene(const bpsx_scene_params *p, uint8_t **out, size_t *out_size);
+BPSX_API int bpsx_gen_scene(const bpsx_scene_params *p, uint8_t **out, size_t *out_size);
 /* Area-weighted random points on the walkable polygons of MSET bytes, host-only:
  * out_xyz f32[n][3]. Deterministic in seed. */
-int bpsx_sample_points(const void *navmesh_bytes, size_t navmesh_size, uint64_t seed,
+BPSX_API int bpsx_sample_points(const void *navmesh_bytes, size_t navmesh_size, uint64_t seed,
                        uint32_t n, float *out_xyz);
 
 #ifdef __cplusplus

@@ -6,6 +6,7 @@ import json
 import os
 import re
 import struct
+import subprocess
 import zlib
 
 import numpy as np
@@ -27,6 +28,11 @@ def test_library_exports_every_declared_symbol():
     L = ctypes.CDLL(_lib.LIB_PATH)
     missing = [n for n in sorted(names) if not hasattr(L, n)]
     assert not missing, f"libbpsx.so lacks {missing}"
+    # ... and nothing else: no C++ internals, no template instantiations (one .so, C ABI only)
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = {ln.split()[-1] for ln in out.splitlines() if ln.strip()}
+    extra = sorted(exported - names)
+    assert not extra, f"libbpsx.so exports symbols that include/bpsx.h does not declare: {extra[:10]}"
 
 
 def test_generator_is_deterministic_and_seed_sensitive():
