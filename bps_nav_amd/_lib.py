@@ -83,6 +83,8 @@ def lib():
             L.bpsx_reset.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p]
             L.bpsx_step_start.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p, C.c_int, C.c_void_p]
             L.bpsx_step_end.argtypes = [C.c_void_p, C.c_uint32]
+            L.bpsx_set_stream_ordered.argtypes = [C.c_void_p, C.c_int]
+            L.bpsx_synchronize.argtypes = [C.c_void_p]
             L.bpsx_get_outputs.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(Outputs)]
             L.bpsx_get_state.argtypes = [C.c_void_p, C.c_uint32, C.POINTER(State)]
             L.bpsx_check_errors.argtypes = [C.c_void_p]

@@ -78,11 +78,12 @@ class PointNavRolloutGenerator:
     def __init__(self, dataset_path, asset_path, num_environments, num_active_scenes, num_workers=-1, gpu_id=0,
                  render_resolution=(64, 64), color=False, depth=False, double_buffered=False, seed=0,
                  should_set_affinity=True, *, scenes=None, reset_mode=0, max_steps=0, scene_reserve=0.0, rotate=None,
-                 rotation_interval_ms=1000):
+                 rotation_interval_ms=1000, stream_ordered=False):
         """`scenes` or the dataset directory may hold more scenes than num_active_scenes: the
         library then picks the ones that start resident at random, on `seed`, and (rotate=True,
         the default for a dataset directory, as in the reference) brings the others in over time,
-        loading at most one scene per rotation_interval_ms in a thread of its own."""
+        loading at most one scene per rotation_interval_ms in a thread of its own.
+        stream_ordered=True: step_end does not wait for the device (see set_stream_ordered)."""
         self._L = _lib.lib()
         if not hasattr(self._L, "bpsx_create"):
             raise RuntimeError("libbpsx.so was built without the HIP engine")
@@ -115,6 +116,8 @@ class PointNavRolloutGenerator:
         self.num_scenes = num_active_scenes
         self._keep = None  # host action array kept alive between step_start and step_end
         self._views = {}
+        if stream_ordered:
+            self.set_stream_ordered(True)
 
     def close(self):
         if getattr(self, "_h", None):
@@ -150,6 +153,17 @@ class PointNavRolloutGenerator:
     def step_end(self, group_idx):
         _lib.check(self._L.bpsx_step_end(self._h, group_idx))
         self._keep = None
+
+    def set_stream_ordered(self, enabled):
+        """Stream-ordered stepping (bpsx_set_stream_ordered): step_end returns without waiting;
+        the outputs are complete for work enqueued afterwards on the stream that was current at
+        step_start (tensor operations on the output tensors, the next step).  Reading them on the
+        host needs synchronize() or a stream synchronization first (`.cpu()` does one)."""
+        _lib.check(self._L.bpsx_set_stream_ordered(self._h, int(bool(enabled))))
+
+    def synchronize(self):
+        """Waits until every step enqueued so far has completed on the device."""
+        _lib.check(self._L.bpsx_synchronize(self._h))
 
     def step(self, group_idx, actions):
         self.step_start(group_idx, actions)

@@ -43,10 +43,23 @@ struct Group {
   hipEvent_t moved = nullptr, snapped = nullptr;   // fork and join of the side stream within a step
   int64_t* d_actions = nullptr;
   int64_t* h_actions = nullptr;  // pinned staging for host-side action arrays
-  hipEvent_t done = nullptr;
   hipEvent_t ev[kStepEvents] = {};
   bool in_flight = false;
   bool profiled = false;
+  int record = -1;               // ring entry of the step in flight
+};
+
+// A step that has been enqueued and whose completion the host has not yet seen.  The host may
+// run ahead of the device by kStepRing steps (stream-ordered stepping, bpsx_set_stream_ordered):
+// what a step brings back for the host (how many envs of each scene slot are still on a scene
+// that is leaving) lands in the step's own pinned buffer and is looked at when its event is
+// found complete.
+constexpr int kStepRing = 4;
+struct StepRecord {
+  hipEvent_t done = nullptr;
+  uint32_t* remaining = nullptr;   // pinned, one word per scene slot
+  uint64_t ordinal = 0;            // sim->steps_started when the step was enqueued
+  bool has_remaining = false;
 };
 
 template <class T>
@@ -128,10 +141,14 @@ struct SceneRanges {
 struct SceneSlot {
   uint32_t current = 0;         // scene-table entry of the resident scene
   uint32_t target = kNoSwap;    // entry of the scene being moved to, if a swap is in progress or just done
+  uint64_t target_ordinal = 0;  // the step that made it the target: earlier steps' counts say nothing about this swap
   // automatic rotation (SceneSwapper, simulator.cpp:1063-1154)
   uint32_t active_scene = 0;    // dataset index of the scene the slot's envs are on or are moving to
   uint32_t load_entry = kNoSwap;          // scene-table entry the loader thread is filling / has filled
   std::atomic<uint32_t> load_state{0};    // 0 none, 1 requested, 2 resident and ready, 3 failed
+  // A slot's two scene-table entries are never touched by both threads at once: the loader
+  // thread writes load_entry's ranges and table entry only between load_state 1 and 2 or 3, the
+  // stepping thread reads or releases them only outside that interval.
 };
 // One scene of the dataset as handed to bpsx_add_scene: kept as bytes while it is not resident.
 struct PoolScene {
@@ -165,6 +182,8 @@ struct bpsx_sim {
   float* d_episodes = nullptr;
   NavData nav{};
   Arena ar_poly, ar_bv, ar_tri, ar_dv, ar_ep;
+  bool fixed_regions = false;        // automatic rotation: one region per scene-table entry instead of the arenas
+  SceneRanges region;                // n*: elements of one region in each array
   std::vector<SceneRanges> ranges;   // per scene-table entry
   std::unique_ptr<SceneSlot[]> slots;
   // dataset and automatic rotation
@@ -179,10 +198,13 @@ struct bpsx_sim {
   std::deque<uint32_t> loader_requests;  // slots waiting for their next scene
   bool loader_exit = false;
   std::string loader_error;              // first failure of the loader thread (guarded by loader_mu)
+  bool loader_error_reported = false;    // step_end has returned it once
   hipStream_t upload_stream = nullptr;   // uploads of scenes that come in while the simulation runs
   hipStream_t side = nullptr;            // a step's snaps of new episodes, next to its searches (default priority)
-  uint32_t* h_swap_remaining = nullptr;  // pinned copy of d_swap_remaining, refreshed by every step
-  bool remaining_fresh = false;
+  uint32_t* h_swap_remaining = nullptr;  // d_swap_remaining as of the newest step whose completion has been seen
+  StepRecord ring[kStepRing];
+  int ring_head = 0, ring_count = 0;     // oldest outstanding record, number outstanding
+  bool stream_ordered = false;           // step_end leaves the waiting to the stream (bpsx_set_stream_ordered)
   std::vector<uint32_t> rotation_log;    // (step ordinal, slot, dataset index) of swaps made available
   uint64_t steps_started = 0, env_steps_taken = 0;
   uint32_t* d_swap_target = nullptr;
@@ -288,7 +310,17 @@ static int upload_scene(bpsx_sim* sim, HostScene& s, uint32_t entry, hipStream_t
   SceneRanges r;
   r.npoly = s.polys.size(); r.nbv = s.bv.size(); r.ntri = s.dtris.size() / 4; r.ndv = s.dverts.size() / 3;
   r.nep = s.episodes.size() / 10;
-  {
+  if (sim->fixed_regions) {
+    // automatic rotation: every scene-table entry owns a region that holds the largest scene of
+    // the pool, so a load can neither fail nor depend on what came and went before it
+    const SceneRanges& m = sim->region;
+    if (r.npoly > m.npoly || r.nbv > m.nbv || r.ntri > m.ntri || r.ndv > m.ndv || r.nep > m.nep)
+      return fail(BPSX_E_UNSUPPORTED, "scene is larger than the largest scene the simulator was finalized with");
+    r.poly = entry * m.npoly; r.bv = entry * m.nbv; r.tri = entry * m.ntri; r.dv = entry * m.ndv; r.ep = entry * m.nep;
+    r.used = true;
+    std::lock_guard<std::mutex> lk(sim->arena_mu);
+    sim->ranges[entry] = r;
+  } else {
     std::lock_guard<std::mutex> lk(sim->arena_mu);
     const bool a = sim->ar_poly.take(r.npoly, &r.poly);
     const bool b = a && sim->ar_bv.take(r.nbv, &r.bv);
@@ -302,12 +334,12 @@ static int upload_scene(bpsx_sim* sim, HostScene& s, uint32_t entry, hipStream_t
       if (d) sim->ar_dv.give(r.dv, r.ndv);
       return fail(BPSX_E_UNSUPPORTED, "scene does not fit the space reserved for scene rotation");
     }
+    r.used = true;
+    sim->ranges[entry] = r;
   }
-  r.used = true;
   s.dev.poly_base = (uint32_t)r.poly; s.dev.bv_base = (uint32_t)r.bv; s.dev.ep_base = (uint32_t)r.ep;
   s.dev.ep_count = (uint32_t)r.nep;
   for (auto& p : s.polys) { p.tri_base += (uint32_t)r.tri; p.dvert_base += (uint32_t)r.dv; }
-  sim->ranges[entry] = r;
   const auto H2D = hipMemcpyHostToDevice;
   HIP_TRY(hipMemcpyAsync(sim->d_polys + r.poly, s.polys.data(), r.npoly * sizeof(PolyRec), H2D, st));
   HIP_TRY(hipMemcpyAsync(sim->d_aedges + r.poly * kEdgeStride, s.aedges.data(), s.aedges.size() * sizeof(AEdge), H2D, st));
@@ -323,6 +355,7 @@ static void release_scene(bpsx_sim* sim, uint32_t entry) {
   std::lock_guard<std::mutex> lk(sim->arena_mu);
   SceneRanges& r = sim->ranges[entry];
   if (!r.used) return;
+  if (sim->fixed_regions) { r = SceneRanges{}; return; }
   sim->ar_poly.give(r.poly, r.npoly); sim->ar_bv.give(r.bv, r.nbv); sim->ar_tri.give(r.tri, r.ntri);
   sim->ar_dv.give(r.dv, r.ndv); sim->ar_ep.give(r.ep, r.nep);
   r = SceneRanges{};
@@ -364,6 +397,7 @@ static void loader_loop(bpsx_sim* sim) {
       rc = upload_scene(sim, hs, sl.load_entry, sim->upload_stream);
     }
     if (rc) {
+      // step_end reports it; the slot keeps its scene and stops rotating
       std::lock_guard<std::mutex> lk(sim->loader_mu);
       if (sim->loader_error.empty())
         sim->loader_error = "scene " + std::to_string(sl.active_scene) + " for slot " + std::to_string(slot) + ": " + last_error_message();
@@ -399,6 +433,7 @@ static int rotation_pre_step(bpsx_sim* sim, hipStream_t st) {
     if (sl.load_state.load(std::memory_order_acquire) != 2) continue;
     sl.load_state.store(0, std::memory_order_relaxed);
     sl.target = sl.load_entry;
+    sl.target_ordinal = sim->steps_started;
     launch_set_swap(sim->d_swap_target, sim->d_swap_remaining, slot, sl.target, per, st);
     HIP_TRY(hipGetLastError());
     sim->h_swap_remaining[slot] = per;
@@ -409,18 +444,44 @@ static int rotation_pre_step(bpsx_sim* sim, hipStream_t st) {
   return BPSX_OK;
 }
 // SceneSwapper::postStep: a slot whose envs have all moved gives its old scene's space back and
-// starts loading its next scene.
-static void rotation_post_step(bpsx_sim* sim) {
+// starts loading its next scene.  `rec` is a step that has completed: its counts are what the
+// device held after it.  Steps enqueued after it do not read the old scene either (every env of
+// the slot had left it), so its space can go to the loader at once.
+static void rotation_post_step(bpsx_sim* sim, const StepRecord& rec) {
   const uint32_t S = sim->cfg.num_active_scenes;
   for (uint32_t slot = 0; slot < S; ++slot) {
     SceneSlot& sl = sim->slots[slot];
-    if (sl.target == kNoSwap || sl.target == sl.current || sim->h_swap_remaining[slot] != 0) continue;
+    if (sl.target == kNoSwap || sl.target == sl.current || sl.target_ordinal > rec.ordinal) continue;
+    sim->h_swap_remaining[slot] = rec.remaining[slot];
+    if (rec.remaining[slot] != 0) continue;
     release_scene(sim, sl.current);
     sl.current = sl.target;   // the device keeps the target: envs already on it ignore it
     sim->swaps_completed++;
     if (sim->rotating) start_scene_swap(sim, slot);
   }
 }
+
+// Takes the records whose steps have completed off the ring, oldest first.  wait_for: number of
+// records that must leave, waiting for their events if need be (ring_count: all of them).
+static int retire_steps(bpsx_sim* sim, int wait_for) {
+  while (sim->ring_count > 0) {
+    StepRecord& rec = sim->ring[sim->ring_head];
+    if (wait_for > 0) {
+      HIP_TRY(hipEventSynchronize(rec.done));
+    } else {
+      const hipError_t q = hipEventQuery(rec.done);
+      if (q == hipErrorNotReady) break;
+      if (q != hipSuccess) return fail(BPSX_E_HIP, std::string("hipEventQuery: ") + hipGetErrorString(q));
+    }
+    if (rec.has_remaining && sim->rotating) rotation_post_step(sim, rec);
+    sim->ring_head = (sim->ring_head + 1) % kStepRing;
+    sim->ring_count--;
+    wait_for--;
+  }
+  return BPSX_OK;
+}
+// Everything enqueued by earlier steps has completed when this returns.
+static int quiesce(bpsx_sim* sim) { return retire_steps(sim, sim->ring_count); }
 
 int bpsx_finalize(bpsx_sim* sim) {
   if (!sim) return fail(BPSX_E_INVAL, "finalize: null simulator");
@@ -445,23 +506,30 @@ int bpsx_finalize(bpsx_sim* sim) {
     sim->slots.reset(new SceneSlot[S]);
     for (uint32_t k = 0; k < S; ++k) sim->slots[k].active_scene = active[k];
   }
-  // ---- navmesh arrays: every scene is a range of each array; room for scene rotation
-  size_t npoly = 0, nbv = 0, ntri = 0, ndv = 0, nep = 0, mpoly = 0, mbv = 0, mtri = 0, mdv = 0, mep = 0;
-  for (uint32_t k = 0; k < S; ++k) {
-    const HostScene& s = *sim->pool[sim->slots[k].active_scene].parsed;
-    npoly += s.polys.size(); nbv += s.bv.size(); ntri += s.dtris.size() / 4; ndv += s.dverts.size() / 3;
-    nep += s.episodes.size() / 10;
-  }
-  for (auto& ps : sim->pool) {   // any scene of the dataset may come in later
-    const HostScene& s = *ps.parsed;
-    mpoly = std::max(mpoly, s.polys.size()); mbv = std::max(mbv, s.bv.size()); mtri = std::max(mtri, s.dtris.size() / 4);
-    mdv = std::max(mdv, s.dverts.size() / 3); mep = std::max(mep, s.episodes.size() / 10);
-  }
+  // ---- navmesh arrays: every scene is a range of each array.
+  // Without automatic rotation the scenes lie one after the other, with room for scenes that the
+  // caller may swap in (bpsx_swap_scene; their sizes are not known: scene_reserve times the
+  // initial scenes plus the largest one, handed out first-fit).  With automatic rotation any
+  // scene of the pool may become resident, two per slot while a swap is in progress, in any
+  // order: each of the 2 S scene-table entries owns a region as large as the largest scene of
+  // the pool, so that no sequence of swaps can fail for lack of a free range of the right size
+  // (S = 128 mazes of 32k polygons: 2.4 GB of the GPU's 288).
+  const bool will_rotate = sim->cfg.rotate_scenes && !sim->inactive.empty();
   const double k = sim->cfg.scene_reserve > 0 ? (double)sim->cfg.scene_reserve : 3.0;
   if (k < 1.0) return fail(BPSX_E_INVAL, "finalize: scene_reserve must be at least 1");
-  auto room = [k](size_t total, size_t largest) { return (size_t)((double)total * k) + largest + 64; };
-  const size_t cpoly = room(npoly, mpoly), cbv = room(nbv, mbv), ctri = room(ntri, mtri), cdv = room(ndv, mdv),
-               cep = room(nep, mep);
+  auto capacity = [&](auto size_of, size_t* region) {
+    size_t total = 0, largest = 0;
+    for (uint32_t i = 0; i < S; ++i) total += size_of(*sim->pool[sim->slots[i].active_scene].parsed);
+    for (auto& ps : sim->pool) largest = std::max(largest, (size_t)size_of(*ps.parsed));
+    *region = largest;
+    return will_rotate ? 2 * (size_t)S * largest + 64 : (size_t)((double)total * k) + largest + 64;
+  };
+  sim->fixed_regions = will_rotate;
+  const size_t cpoly = capacity([](const HostScene& s) { return s.polys.size(); }, &sim->region.npoly);
+  const size_t cbv = capacity([](const HostScene& s) { return s.bv.size(); }, &sim->region.nbv);
+  const size_t ctri = capacity([](const HostScene& s) { return s.dtris.size() / 4; }, &sim->region.ntri);
+  const size_t cdv = capacity([](const HostScene& s) { return s.dverts.size() / 3; }, &sim->region.ndv);
+  const size_t cep = capacity([](const HostScene& s) { return s.episodes.size() / 10; }, &sim->region.nep);
   if (cpoly > 0xfffffff0ull || ctri > 0xfffffff0ull) return fail(BPSX_E_UNSUPPORTED, "finalize: navmeshes too large");
   int rc;
   if ((rc = sim->alloc(&sim->d_polys, cpoly))) return rc;
@@ -483,12 +551,17 @@ int bpsx_finalize(bpsx_sim* sim) {
   HIP_TRY(hipStreamCreateWithFlags(&sim->side, hipStreamNonBlocking));
   HIP_TRY(hipHostMalloc((void**)&sim->h_swap_remaining, (size_t)S * 4, hipHostMallocDefault));
   memset(sim->h_swap_remaining, 0, (size_t)S * 4);
+  for (StepRecord& rec : sim->ring) {
+    HIP_TRY(hipEventCreateWithFlags(&rec.done, hipEventDisableTiming));
+    HIP_TRY(hipHostMalloc((void**)&rec.remaining, (size_t)S * 4, hipHostMallocDefault));
+    memset(rec.remaining, 0, (size_t)S * 4);
+  }
   for (uint32_t i = 0; i < S; ++i) {
     sim->slots[i].current = i;
     if ((rc = upload_scene(sim, *sim->pool[sim->slots[i].active_scene].parsed, i, sim->upload_stream))) return rc;
   }
   // the parsed copies are not needed any more; the bytes stay only if scenes will rotate
-  sim->rotating = sim->cfg.rotate_scenes && !sim->inactive.empty();
+  sim->rotating = will_rotate;
   for (auto& ps : sim->pool) {
     ps.parsed.reset();
     if (!sim->rotating) { ps.blob.clear(); ps.blob.shrink_to_fit(); ps.episodes.clear(); ps.episodes.shrink_to_fit(); }
@@ -549,7 +622,6 @@ int bpsx_finalize(bpsx_sim* sim) {
     HIP_TRY(hipEventCreateWithFlags(&g.moved, hipEventDisableTiming));
     HIP_TRY(hipEventCreateWithFlags(&g.snapped, hipEventDisableTiming));
     HIP_TRY(hipHostMalloc((void**)&g.h_actions, n * sizeof(int64_t), hipHostMallocDefault));
-    HIP_TRY(hipEventCreateWithFlags(&g.done, hipEventDisableTiming));
     for (auto& e : g.ev) HIP_TRY(hipEventCreate(&e));
   }
   // the allocation-free entry point's scratch: its address on this device, looked up here so
@@ -581,9 +653,12 @@ void bpsx_destroy(bpsx_sim* sim) {
   if (sim->upload_stream) (void)hipStreamDestroy(sim->upload_stream);
   if (sim->side) (void)hipStreamDestroy(sim->side);
   if (sim->h_swap_remaining) (void)hipHostFree(sim->h_swap_remaining);
+  for (StepRecord& rec : sim->ring) {
+    if (rec.done) (void)hipEventDestroy(rec.done);
+    if (rec.remaining) (void)hipHostFree(rec.remaining);
+  }
   for (auto& g : sim->groups) {
     if (g.h_actions) (void)hipHostFree(g.h_actions);
-    if (g.done) (void)hipEventDestroy(g.done);
     if (g.moved) (void)hipEventDestroy(g.moved);
     if (g.snapped) (void)hipEventDestroy(g.snapped);
     for (auto& e : g.ev)
@@ -613,6 +688,7 @@ int bpsx_reset(bpsx_sim* sim, uint32_t group, void* hip_stream) {
   Group& g = sim->groups[group];
   if (g.in_flight) return fail(BPSX_E_STATE, "reset: a step of this group is still in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  if ((rc = quiesce(sim))) return rc;
   hipStream_t st = (hipStream_t)hip_stream;
   launch_reset(sim->nav, sim->A, g.Q[g.turn], g.Q[g.turn ^ 1], sim->params(group), sim->d_slots, sim->geo_blocks, sim->snap_blocks, st);
   HIP_TRY(hipGetLastError());
@@ -630,8 +706,12 @@ int bpsx_step_start(bpsx_sim* sim, uint32_t group, const int64_t* actions, int a
     if (og.in_flight) return fail(BPSX_E_STATE, "step_start: previous step not finished (call step_end first)");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
   hipStream_t st = (hipStream_t)hip_stream;
+  // steps that have completed leave the ring; a full ring makes the host wait for its oldest step
+  if ((rc = retire_steps(sim, sim->ring_count == kStepRing ? 1 : 0))) return rc;
   const int64_t* d_act = actions;
   if (!actions_on_device) {
+    // the staging buffer may still be waiting to be read by a step that has not run yet
+    if ((rc = quiesce(sim))) return rc;
     memcpy(g.h_actions, actions, (size_t)sim->envs_per_group * sizeof(int64_t));
     HIP_TRY(hipMemcpyAsync(g.d_actions, g.h_actions, (size_t)sim->envs_per_group * sizeof(int64_t), hipMemcpyHostToDevice, st));
     d_act = g.d_actions;
@@ -644,14 +724,17 @@ int bpsx_step_start(bpsx_sim* sim, uint32_t group, const int64_t* actions, int a
               sim->side, g.moved, g.snapped, g.profiled ? g.ev : nullptr);
   g.turn ^= 1;
   HIP_TRY(hipGetLastError());
+  g.record = (sim->ring_head + sim->ring_count) % kStepRing;
+  StepRecord& rec = sim->ring[g.record];
+  rec.ordinal = sim->steps_started;
   // how many envs of each slot are still on a scene that is leaving: read back with the step
-  sim->remaining_fresh = false;
-  for (uint32_t slot = 0; slot < sim->cfg.num_active_scenes && !sim->remaining_fresh; ++slot)
-    sim->remaining_fresh = sim->slots[slot].target != kNoSwap && sim->slots[slot].target != sim->slots[slot].current;
-  if (sim->remaining_fresh)
-    HIP_TRY(hipMemcpyAsync(sim->h_swap_remaining, sim->d_swap_remaining, (size_t)sim->cfg.num_active_scenes * 4,
-                           hipMemcpyDeviceToHost, st));
-  HIP_TRY(hipEventRecord(g.done, st));
+  rec.has_remaining = false;
+  for (uint32_t slot = 0; slot < sim->cfg.num_active_scenes && !rec.has_remaining; ++slot)
+    rec.has_remaining = sim->slots[slot].target != kNoSwap && sim->slots[slot].target != sim->slots[slot].current;
+  if (rec.has_remaining)
+    HIP_TRY(hipMemcpyAsync(rec.remaining, sim->d_swap_remaining, (size_t)sim->cfg.num_active_scenes * 4, hipMemcpyDeviceToHost, st));
+  HIP_TRY(hipEventRecord(rec.done, st));
+  sim->ring_count++;
   g.in_flight = true;
   sim->steps_started++;
   sim->env_steps_taken += sim->envs_per_group;
@@ -664,9 +747,11 @@ int bpsx_step_end(bpsx_sim* sim, uint32_t group) {
   Group& g = sim->groups[group];
   // the reference aborts with "Simulation already done" / group mismatch (simulator.cpp:1679-1689)
   if (!g.in_flight) return fail(BPSX_E_STATE, "step_end: no step in flight for this group");
-  HIP_TRY(hipEventSynchronize(g.done));
+  // Host-synchronous stepping waits for the step here.  Stream-ordered stepping does not: the
+  // step's outputs are complete for whatever is enqueued next on the stream step_start was
+  // given, and the host only looks at what earlier steps have brought back.
+  if ((rc = retire_steps(sim, (sim->stream_ordered && !g.profiled) ? 0 : sim->ring_count))) return rc;
   g.in_flight = false;
-  if (sim->remaining_fresh && sim->rotating) rotation_post_step(sim);
   if (g.profiled) {
     for (int k = 0; k < BPSX_NUM_KERNELS; ++k) {
       float ms = 0;
@@ -675,7 +760,30 @@ int bpsx_step_end(bpsx_sim* sim, uint32_t group) {
     }
     sim->profiled_steps++;
   }
+  if (sim->rotating && !sim->loader_error_reported) {
+    // a scene that could not be loaded (the reference aborts, simulator.cpp:1723-1726): the step
+    // itself is complete, its slot keeps its scene and stops rotating
+    std::lock_guard<std::mutex> lk(sim->loader_mu);
+    if (!sim->loader_error.empty()) {
+      sim->loader_error_reported = true;
+      return fail(BPSX_E_UNSUPPORTED, "step_end: scene rotation: loading failed: " + sim->loader_error);
+    }
+  }
   return BPSX_OK;
+}
+
+int bpsx_set_stream_ordered(bpsx_sim* sim, int enabled) {
+  if (!sim) return fail(BPSX_E_INVAL, "set_stream_ordered: null simulator");
+  for (auto& g : sim->groups)
+    if (g.in_flight) return fail(BPSX_E_STATE, "set_stream_ordered: a step is in flight");
+  sim->stream_ordered = enabled != 0;
+  return BPSX_OK;
+}
+
+int bpsx_synchronize(bpsx_sim* sim) {
+  if (!sim || !sim->finalized) return fail(BPSX_E_STATE, "synchronize: simulator not finalized");
+  HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  return quiesce(sim);
 }
 
 int bpsx_get_outputs(bpsx_sim* sim, uint32_t group, bpsx_outputs* out) {
@@ -711,6 +819,7 @@ int bpsx_get_state(bpsx_sim* sim, uint32_t group, bpsx_state* out) {
 
 int bpsx_check_errors(bpsx_sim* sim) {
   if (!sim || !sim->finalized) return fail(BPSX_E_STATE, "check_errors: simulator not finalized");
+  { const int qrc = quiesce(sim); if (qrc) return qrc; }
   uint32_t f = 0;
   HIP_TRY(hipMemcpy(&f, sim->d_error, 4, hipMemcpyDeviceToHost));
   if (f) return fail(BPSX_E_ACTION, "an action id outside 0..3 was passed to step");
@@ -719,6 +828,7 @@ int bpsx_check_errors(bpsx_sim* sim) {
 
 int bpsx_get_counters(bpsx_sim* sim, uint64_t* out) {
   if (!sim || !sim->finalized || !out) return fail(BPSX_E_STATE, "get_counters: simulator not finalized");
+  { const int qrc = quiesce(sim); if (qrc) return qrc; }
   HIP_TRY(hipMemcpy(out, sim->d_counters, BPSX_NUM_COUNTERS * 8, hipMemcpyDeviceToHost));
   return BPSX_OK;
 }
@@ -783,6 +893,7 @@ int bpsx_swap_scene(bpsx_sim* sim, uint32_t slot, const void* navmesh_bytes, siz
     if (g.in_flight) return fail(BPSX_E_STATE, "swap_scene: a step is in flight");
   if (sim->rotating) return fail(BPSX_E_STATE, "swap_scene: this simulator rotates its scenes by itself");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  { const int qrc = quiesce(sim); if (qrc) return qrc; }
   // no step is in flight and every earlier one was waited for in step_end: nothing reads the
   // scene that may leave now, and the upload below runs on a stream of its own
   uint32_t remaining = 0;
@@ -809,6 +920,7 @@ int bpsx_swap_status(bpsx_sim* sim, uint32_t slot, uint32_t* envs_remaining, uin
   for (auto& g : sim->groups)
     if (g.in_flight) return fail(BPSX_E_STATE, "swap_status: a step is in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
+  { const int qrc = quiesce(sim); if (qrc) return qrc; }
   uint32_t remaining = 0;
   if (sim->rotating) {
     // as of the last step (step_end keeps the count and completes swaps by itself)
@@ -882,13 +994,15 @@ static uint32_t scene_entry(const bpsx_sim* sim, uint32_t slot) {
   return sl.target != kNoSwap ? sl.target : sl.current;
 }
 
-static int check_scene(bpsx_sim* sim, uint32_t scene, const char* what) {
+// wait: the call reads results back on the host, so steps still running on the device are waited
+// for first (stream-ordered stepping leaves them running after step_end)
+static int check_scene(bpsx_sim* sim, uint32_t scene, const char* what, bool wait = true) {
   if (!sim || !sim->finalized) return fail(BPSX_E_STATE, std::string(what) + ": simulator not finalized");
   if (scene >= sim->cfg.num_active_scenes) return fail(BPSX_E_INVAL, std::string(what) + ": scene out of range");
   for (auto& g : sim->groups)
     if (g.in_flight) return fail(BPSX_E_STATE, std::string(what) + ": a step is in flight");
   HIP_TRY(hipSetDevice(sim->cfg.gpu_id));
-  return BPSX_OK;
+  return wait ? quiesce(sim) : BPSX_OK;
 }
 
 int bpsx_snap_points(bpsx_sim* sim, uint32_t scene, const float* pts, uint32_t n, float* out_xyz, uint32_t* out_ref) {
@@ -955,7 +1069,7 @@ int bpsx_geodesic(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const u
 
 int bpsx_geodesic_static(bpsx_sim* sim, uint32_t scene, const float* start_xyz, const uint32_t* start_ref,
                          const float* end_xyz, const uint32_t* end_ref, uint32_t n, float* out_dist, void* hip_stream) {
-  int rc = check_scene(sim, scene, "geodesic_static");
+  int rc = check_scene(sim, scene, "geodesic_static", false);   // stream-ordered: nothing is waited for
   if (rc) return rc;
   if (n > BPSX_STATIC_MAX_QUERIES)
     return fail(BPSX_E_INVAL, "geodesic_static: n = " + std::to_string(n) + " exceeds BPSX_STATIC_MAX_QUERIES = " +

@@ -173,8 +173,25 @@ BPSX_API int bpsx_reset(bpsx_sim *sim, uint32_t group, void *hip_stream);
  * step on): outputs and state arrays are the same after every step. */
 BPSX_API int bpsx_step_start(bpsx_sim *sim, uint32_t group, const int64_t *actions,
                     int actions_on_device, void *hip_stream);
-/* step_end(group): waits until the step's outputs are complete. */
+/* step_end(group): waits until the step's outputs are complete (host-synchronous stepping, the
+ * default), or returns at once (stream-ordered stepping, below).  Returns BPSX_E_UNSUPPORTED once,
+ * with the step complete, when the scene rotation's loader thread could not load a scene (the
+ * reference aborts, simulator.cpp:1723-1726); that slot keeps its scene from then on. */
 BPSX_API int bpsx_step_end(bpsx_sim *sim, uint32_t group);
+/* Stream-ordered stepping ("step_end = no-op if the consumer is stream-ordered"): with
+ * enabled != 0, step_end does not wait for the device.  The step's outputs are complete for
+ * everything enqueued afterwards on the stream that step_start was given (device-to-device
+ * copies into a rollout storage, the policy's kernels, the next step_start), and a consumer on
+ * the host calls bpsx_synchronize (or synchronizes that stream) before it reads them.  The host
+ * may run up to four steps ahead of the device; step_start waits for the oldest of them when it
+ * would be more.  Host-side action arrays (actions_on_device == 0) make step_start wait for all
+ * earlier steps; while per-kernel timing is on, step_end waits as in the default mode.  Entry
+ * points that bring results to the host (reset, the batched queries, counters, errors, swap
+ * status) wait for outstanding steps by themselves.  The one-outstanding-step rule
+ * (simulator.cpp:1659-1662, 1679-1689) is unchanged: step_start, step_end, step_start, ... */
+BPSX_API int bpsx_set_stream_ordered(bpsx_sim *sim, int enabled);
+/* Waits until every step enqueued so far has completed on the device. */
+BPSX_API int bpsx_synchronize(bpsx_sim *sim);
 BPSX_API int bpsx_get_outputs(bpsx_sim *sim, uint32_t group, bpsx_outputs *out);
 BPSX_API int bpsx_get_state(bpsx_sim *sim, uint32_t group, bpsx_state *out);
 /* Sticky error flag raised by kernels (invalid action ids): 0 or BPSX_E_ACTION. */

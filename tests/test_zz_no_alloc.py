@@ -47,6 +47,44 @@ def test_static_geodesic_matches_the_allocating_entry_point(oracle):
                 ref = nav.geodesic(a[:500], ar[:500], b[:500], br[:500])
                 assert np.array_equal(common.bits(ref), common.bits(got[:500])), "differs from the oracle"
         nav.close()
+    # ---- what the entry point is for: no allocation, and usable under stream capture
+    blob = blobs[1]
+    pts = scenes.sample_points(blob, 99, 2 * 500)
+    x, r = gen.snap_points(1, pts)
+    t = lambda v, dt: torch.from_numpy(np.ascontiguousarray(v).view(dt)).cuda()  # noqa: E731
+    a, ar, b, br = t(x[:500], np.float32), t(r[:500], np.int32), t(x[500:], np.float32), t(r[500:], np.int32)
+    want = gen.geodesic(1, x[:500], r[:500], x[500:], r[500:])
+    out = torch.full((500,), -1.0, device="cuda")
+    gen.geodesic_static(1, a, ar, b, br, out=out)           # warm: everything the call touches exists
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    reserved0 = torch.cuda.memory_reserved()
+    for _ in range(3):
+        gen.geodesic_static(1, a, ar, b, br, out=out)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "device memory in use changed across allocation-free calls"
+    assert torch.cuda.memory_reserved() == reserved0
+    assert np.array_equal(common.bits(want), common.bits(out.cpu().numpy()))
+    # captured once into a HIP graph, replayed three times with eager work and synchronizations in
+    # between and other inputs in the same buffers: every replay equals the allocating entry point
+    graph = torch.cuda.CUDAGraph()
+    out.fill_(-1.0)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        gen.geodesic_static(1, a, ar, b, br, out=out)
+    for rep in range(3):
+        perm = np.random.default_rng(rep).permutation(500)
+        xa, ra = x[:500][perm], r[:500][perm]
+        a.copy_(t(xa, np.float32))
+        ar.copy_(t(ra, np.int32))
+        want = gen.geodesic(1, xa, ra, x[500:], r[500:])    # eager work of the library between replays
+        out.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.array_equal(common.bits(want), common.bits(got)), f"graph replay {rep} differs"
+    del graph
     # limits and empty input
     z3 = torch.zeros((gen.STATIC_MAX_QUERIES + 1, 3), device="cuda")
     zr = torch.zeros(gen.STATIC_MAX_QUERIES + 1, dtype=torch.int32, device="cuda")
