@@ -514,8 +514,8 @@ BPSX_DEV void serve_query(Wave& g, const NavData& nav, const GeoQuery& q, int cl
   const unsigned long long trace_pred = (last_cost && q.cost_slot != kNoCostSlot) ? last_cost[q.cost_slot] : 0xffffu;
 #endif
   // the longer the expected search, the sooner its instructions issue; a search of unknown
-  // length may be among the longest
-  set_wave_priority(cls == (int)kGeoClassUnknown ? 3 : (int)(((uint32_t)(kGeoClasses - 1 - cls) * kGeoClassWidth) / 400u));
+  // length may be among the longest, but most are not: they run just below those known to be long
+  set_wave_priority(cls == (int)kGeoClassUnknown ? 2 : (int)(((uint32_t)(kGeoClasses - 1 - cls) * kGeoClassWidth) / 400u));
   const float d = geodesic_query(g, nav, q, &T.pops, &T.corridor);
   if (g.lane == 0) {
 #ifdef BPSX_QUERY_TRACE

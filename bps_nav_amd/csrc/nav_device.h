@@ -339,6 +339,118 @@ BPSX_DEV NavPt snap_point_wave(const NavData& nav, const SceneDev& s, float px, 
   return out;
 }
 
+// A polygon record in registers, for the move of one agent per lane: its first 112 bytes arrive
+// with seven 16-byte loads that go out together, where the loops over a record in memory pay a
+// load and a wait for every field as they come to it (a forward move is one chain of dependent
+// loads: state, scene, polygon, neighbour polygon, height mesh).  Every index into the words is
+// a compile-time constant (loops over vertices are unrolled in the source, through static_for,
+// not left to the optimiser: an index that is still a loop variable when the array is looked at
+// sends the record to scratch memory); a vertex or neighbour code with a run-time index is
+// picked by a chain of selects.  Same float operations in the same order as the versions on
+// records in memory above.
+// (lambdas handed to static_for are marked BPSX_INLINE_LAMBDA: inlined together with the functions
+// around them, before the optimiser first looks at the record)
+#define BPSX_INLINE_LAMBDA __attribute__((always_inline))
+template <int I> struct Idx { static constexpr int value = I; };
+template <int B, int E, class F> BPSX_DEV void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(Idx<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+struct PolyRegs {
+  uint32_t w[28];
+  BPSX_DEV void load(const PolyRec* p) {
+    const uint4* s = reinterpret_cast<const uint4*>(p);
+    static_for<0, 7>([&](auto K) BPSX_INLINE_LAMBDA {
+      constexpr int k = decltype(K)::value;
+      const uint4 q = s[k];
+      w[4 * k] = q.x; w[4 * k + 1] = q.y; w[4 * k + 2] = q.z; w[4 * k + 3] = q.w;
+    });
+  }
+  static_assert(offsetof(PolyRec, nei) == 72 && offsetof(PolyRec, walk) == 84 && offsetof(PolyRec, flags) == 96 &&
+                offsetof(PolyRec, nv) == 98 && offsetof(PolyRec, type) == 99 && offsetof(PolyRec, tri_base) == 100 &&
+                offsetof(PolyRec, dvert_base) == 104 && offsetof(PolyRec, tri_count) == 108, "PolyRegs follows PolyRec's layout");
+  template <int I> BPSX_DEV float x() const { return __uint_as_float(w[3 * I]); }
+  template <int I> BPSX_DEV float y() const { return __uint_as_float(w[3 * I + 1]); }
+  template <int I> BPSX_DEV float z() const { return __uint_as_float(w[3 * I + 2]); }
+  template <int J> BPSX_DEV uint32_t nei() const { return (w[18 + (J >> 1)] >> (16 * (J & 1))) & 0xffffu; }
+  template <int J> BPSX_DEV uint32_t walk() const { return (w[21 + (J >> 1)] >> (16 * (J & 1))) & 0xffffu; }
+  BPSX_DEV int nv() const { return (int)((w[24] >> 16) & 0xffu); }
+  BPSX_DEV uint32_t type() const { return w[24] >> 24; }
+  BPSX_DEV uint32_t tri_base() const { return w[25]; }
+  BPSX_DEV uint32_t dvert_base() const { return w[26]; }
+  BPSX_DEV int tri_count() const { return (int)(w[27] & 0xffu); }
+  // vertex k, k known at run time only.  The words pass through an empty asm first: selects
+  // between loads of the array would be folded into one load at a selected address, and the
+  // record would have to live in (scratch) memory for it.
+  static BPSX_DEV uint32_t reg(uint32_t v) { asm("" : "+v"(v)); return v; }
+  BPSX_DEV uint32_t word(int k, int stride, int base) const {   // w[base + stride * k], k in 0..5
+    const uint32_t a0 = reg(w[base]), a1 = reg(w[base + stride]), a2 = reg(w[base + 2 * stride]), a3 = reg(w[base + 3 * stride]),
+                   a4 = reg(w[base + 4 * stride]), a5 = reg(w[base + 5 * stride]);
+    return k == 5 ? a5 : k == 4 ? a4 : k == 3 ? a3 : k == 2 ? a2 : k == 1 ? a1 : a0;
+  }
+  BPSX_DEV void vertex(int k, float* o) const {
+    o[0] = __uint_as_float(word(k, 3, 0));
+    o[1] = __uint_as_float(word(k, 3, 1));
+    o[2] = __uint_as_float(word(k, 3, 2));
+  }
+  BPSX_DEV void codes(int k, uint32_t* nei_k, uint32_t* walk_k) const {
+    const uint32_t n = word(k >> 1, 1, 18), wk = word(k >> 1, 1, 21);   // two 16-bit codes per word; k >> 1 in 0..2
+    *nei_k = (n >> (16 * (k & 1))) & 0xffffu;
+    *walk_k = (wk >> (16 * (k & 1))) & 0xffffu;
+  }
+};
+
+BPSX_DEV bool point_in_poly(float px, float pz, const PolyRegs& P) {
+  bool c = false;
+  const int nv = P.nv();
+  float vj[3];
+  P.vertex(nv - 1, vj);
+  float jx = vj[0], jz = vj[2];
+  static_for<0, kNvp>([&](auto I) BPSX_INLINE_LAMBDA {
+    constexpr int i = decltype(I)::value;
+    const float ix = P.x<i>(), iz = P.z<i>();
+    const bool crosses = ((iz > pz) != (jz > pz)) && (px < (jx - ix) * (pz - iz) / (jz - iz) + ix);
+    c ^= (i < nv) && crosses;
+    jx = ix; jz = iz;
+  });
+  return c;
+}
+
+// dtNavMesh::getPolyHeight on a record in registers (`mem`: the same record in memory, for the
+// rare fall-back to the detail edges).  The index words of the first four detail triangles go
+// out together.
+BPSX_DEV bool poly_height(const NavData& nav, const PolyRegs& P, const PolyRec& mem, float px, float py, float pz, float& h) {
+  if (P.type() != 0) return false;
+  if (!point_in_poly(px, pz, P)) return false;
+  const int tc = P.tri_count(), nv = P.nv();
+  const uint32_t* tris = reinterpret_cast<const uint32_t*>(nav.dtris) + P.tri_base();   // four bytes per triangle
+  const uint32_t t0 = 0 < tc ? tris[0] : 0u, t1 = 1 < tc ? tris[1] : 0u, t2 = 2 < tc ? tris[2] : 0u, t3 = 3 < tc ? tris[3] : 0u;
+  auto corner = [&](uint32_t k, float* o) BPSX_INLINE_LAMBDA {
+    if ((int)k < nv) P.vertex((int)k, o);
+    else {
+      const float* d = &nav.dverts[(size_t)(P.dvert_base() + (k - (uint32_t)nv)) * 3];
+      o[0] = d[0]; o[1] = d[1]; o[2] = d[2];
+    }
+  };
+  auto inside = [&](uint32_t t) BPSX_INLINE_LAMBDA {
+    float a[3], b[3], c[3];
+    corner(t & 0xffu, a); corner((t >> 8) & 0xffu, b); corner((t >> 16) & 0xffu, c);
+    return height_on_triangle(px, pz, a, b, c, h);
+  };
+  if (0 < tc && inside(t0)) return true;
+  if (1 < tc && inside(t1)) return true;
+  if (2 < tc && inside(t2)) return true;
+  if (3 < tc && inside(t3)) return true;
+  for (int j = 4; j < tc; ++j)
+    if (inside(tris[j])) return true;
+  float c[3];
+  closest_on_detail_edges<false>(nav, mem, px, py, pz, c);
+  h = c[1];
+  return true;
+}
+
 // The tiny node pool and the queue of moveAlongSurface, one column per lane of a wavefront, in
 // LDS: they are indexed at run time, which in private memory means a trip to scratch (HBM
 // behind the vector caches) per access.  A node enters the queue at most once, so the queue
@@ -366,58 +478,75 @@ BPSX_DEV NavPt try_step(const NavData& nav, const SceneDev& s, const NavPt& star
   const float ddx = ex - start.x, ddy = ey - start.y, ddz = ez - start.z;
   const float sr = sqrtf(ddx * ddx + ddy * ddy + ddz * ddz) / 2.0f + 0.001f;
   const float searchRadSqr = sr * sr;
+  PolyRegs P;
+  uint32_t loaded = kInvalidPoly;   // the polygon P holds
   while (qhead < qtail) {
     const int cur = M.queue[qhead++][lane];
-    const PolyRec& r = nav.polys[s.poly_base + M.node_id[cur][lane]];
+    loaded = M.node_id[cur][lane];
+    P.load(&nav.polys[s.poly_base + loaded]);
     (*npolys)++;
-    if (point_in_poly(ex, ez, r)) {
+    if (point_in_poly(ex, ez, P)) {
       bestNode = cur;
       bx = ex; by = ey; bz = ez;
       break;
     }
-    const int nv = r.nv;
-    for (int i = 0, j = nv - 1; i < nv; j = i++) {
-      // single-tile meshes carry no tile-border links, so a border edge is a wall
-      const uint16_t nb = (r.nei[j] & 0x8000) ? (uint16_t)0 : r.walk[j];
-      const float* vj = r.v[j];
-      const float* vi = r.v[i];
-      if (!nb) {
-        float t;
-        const float d = dist_pt_seg_sqr2d(ex, ez, vj, vi, t);
-        if (d < bestDist) {
-          bx = vj[0] + (vi[0] - vj[0]) * t;
-          by = vj[1] + (vi[1] - vj[1]) * t;
-          bz = vj[2] + (vi[2] - vj[2]) * t;
-          bestDist = d;
-          bestNode = cur;
-        }
-      } else {
-        const uint16_t ip = (uint16_t)(nb - 1);
-        int nn = -1;
-        for (int k = 0; k < nnodes; ++k)
-          if (M.node_id[k][lane] == ip) { nn = k; break; }
-        if (nn < 0) {
-          if (nnodes >= kTinyNodes) continue;
-          nn = nnodes++;
-          M.node_id[nn][lane] = ip;
-        }
-        if ((closed >> nn) & 1ull) continue;
-        float t;
-        const float d = dist_pt_seg_sqr2d(sx, sz, vj, vi, t);
-        if (d > searchRadSqr) continue;
-        if (qtail - qhead < kMoveQueue) {
-          closed |= 1ull << nn;
-          M.queue[qtail++][lane] = (uint8_t)nn;
+    const int nv = P.nv();
+    // edge j -> i with j the vertex before i: (nv - 1, 0), (0, 1), ...
+    float vj[3];
+    uint32_t neij, walkj;
+    P.vertex(nv - 1, vj);
+    P.codes(nv - 1, &neij, &walkj);
+    static_for<0, kNvp>([&](auto I) BPSX_INLINE_LAMBDA {
+      constexpr int i = decltype(I)::value;
+      const float vi[3] = {P.x<i>(), P.y<i>(), P.z<i>()};
+      if (i < nv) {
+        // single-tile meshes carry no tile-border links, so a border edge is a wall
+        const uint32_t nb = (neij & 0x8000u) ? 0u : walkj;
+        if (!nb) {
+          float t;
+          const float d = dist_pt_seg_sqr2d(ex, ez, vj, vi, t);
+          if (d < bestDist) {
+            bx = vj[0] + (vi[0] - vj[0]) * t;
+            by = vj[1] + (vi[1] - vj[1]) * t;
+            bz = vj[2] + (vi[2] - vj[2]) * t;
+            bestDist = d;
+            bestNode = cur;
+          }
+        } else {
+          const uint16_t ip = (uint16_t)(nb - 1);
+          int nn = -1;
+          for (int k = 0; k < nnodes; ++k)
+            if (M.node_id[k][lane] == ip) { nn = k; break; }
+          bool fits = true;
+          if (nn < 0) {
+            if (nnodes >= kTinyNodes) fits = false;
+            else {
+              nn = nnodes++;
+              M.node_id[nn][lane] = ip;
+            }
+          }
+          if (fits && !((closed >> nn) & 1ull)) {
+            float t;
+            const float d = dist_pt_seg_sqr2d(sx, sz, vj, vi, t);
+            if (!(d > searchRadSqr) && qtail - qhead < kMoveQueue) {
+              closed |= 1ull << nn;
+              M.queue[qtail++][lane] = (uint8_t)nn;
+            }
+          }
         }
       }
-    }
+      vj[0] = vi[0]; vj[1] = vi[1]; vj[2] = vi[2];
+      neij = P.nei<i>(); walkj = P.walk<i>();
+    });
   }
   if (bestNode < 0) return start;
   const uint32_t bestIp = M.node_id[bestNode][lane];
   NavPt out{bx, by, bz, s.ref_base | bestIp};
   if (isfinite(bx) && isfinite(bz)) {
+    const PolyRec& mem = nav.polys[s.poly_base + bestIp];
+    if (bestIp != loaded) P.load(&mem);
     float h;
-    if (poly_height(nav, nav.polys[s.poly_base + bestIp], bx, by, bz, h)) out.y = h;
+    if (poly_height(nav, P, mem, bx, by, bz, h)) out.y = h;
   }
   return out;
 }
