@@ -343,11 +343,12 @@ BPSX_DEV NavPt snap_point_wave(const NavData& nav, const SceneDev& s, float px, 
 // with seven 16-byte loads that go out together, where the loops over a record in memory pay a
 // load and a wait for every field as they come to it (a forward move is one chain of dependent
 // loads: state, scene, polygon, neighbour polygon, height mesh).  Every index into the words is
-// a compile-time constant (loops over vertices are unrolled in the source, through static_for,
-// not left to the optimiser: an index that is still a loop variable when the array is looked at
-// sends the record to scratch memory); a vertex or neighbour code with a run-time index is
-// picked by a chain of selects.  Same float operations in the same order as the versions on
-// records in memory above.
+// a compile-time constant: loops over vertices are unrolled in the source (static_for), and a
+// vertex or neighbour code with a run-time index is picked by a chain of selects whose operands
+// the optimiser cannot trace back to the array (PolyRegs::reg), because either an index that
+// is still a loop variable or a select between two loads of the array makes it an array in
+// scratch memory again.  Same float operations in the same order as the versions on records
+// in memory above.
 // (lambdas handed to static_for are marked BPSX_INLINE_LAMBDA: inlined together with the functions
 // around them, before the optimiser first looks at the record)
 #define BPSX_INLINE_LAMBDA __attribute__((always_inline))

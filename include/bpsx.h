@@ -79,8 +79,10 @@ typedef struct bpsx_config {
   int32_t gpu_id;             /* HIP device ordinal                                        */
   uint32_t max_steps;         /* 0 => BPSX_MAX_STEPS                                       */
   uint32_t task;              /* BPSX_TASK_*                                               */
-  float scene_reserve;        /* space for scene rotation: capacity of the navmesh arrays as
-                                 a multiple of the initial scenes' total size; 0 => 3      */
+  float scene_reserve;        /* space for scenes that bpsx_swap_scene brings in: capacity of the
+                                 navmesh arrays as a multiple of the initial scenes' total size;
+                                 0 => 3.  Not used with rotate_scenes, which sizes the arrays
+                                 from the scenes that were added (see below)               */
   uint32_t rotate_scenes;     /* 1 => when more scenes were added than are resident, rotate
                                  through them by itself (SceneSwapper, simulator.cpp:1063-1154) */
   uint32_t rotation_interval_ms; /* least time between two scene loads of the loader thread
@@ -148,6 +150,10 @@ BPSX_API int bpsx_swap_status(bpsx_sim *sim, uint32_t slot, uint32_t *envs_remai
  * step_start makes a scene that has become resident the slot's target, step_end frees the old
  * scene once every env has left it and draws the slot's next scene uniformly from the scenes
  * that are not resident (startSceneSwap / preStep / postStep, simulator.cpp:1093-1128).
+ * Each slot owns two regions of the navmesh arrays, each as large as the largest scene that was
+ * added (the scene its envs are on and the one they are moving to), so a load never fails for
+ * lack of room, whichever scenes happened to start resident.  A scene that cannot be loaded for
+ * another reason is reported by the next step_end (and by rotation_log); its slot keeps its scene.
  * bpsx_swap_scene is refused on such a simulator.
  * active_scenes: dataset index of the scene each slot's envs are on or are moving to.
  * rotation_log: rows {ordinal of the step_start that made the scene the slot's target, slot,
