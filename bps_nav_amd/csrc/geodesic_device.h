@@ -44,7 +44,10 @@ namespace bpsx {
 #ifdef BPSX_PHASE_TIMING
 // diagnostic build: cycles per phase of the sorted-list loop -> counters: 0 front of the list, 1 fetch, 2 lookup,
 // 3 costs, 4 rows that stand, 5 closing, new nodes and stores, 6 list and log; 7 counts the passes
+// (the comment that the asm statement leaves in the compiler's assembly output names the loop's
+// instantiation and the mark, for tests/measure_astar_loop_phases.py)
 #define FM(k) do { constexpr int slot_[11] = {7, 0, 1, 2, 3, 4, 5, 5, 5, 6, 6}; const unsigned long long now_ = __builtin_readcyclecounter(); \
+    asm volatile("; astar_fast spill=%0 pairs=%1 mark=%2" :: "i"((int)S), "i"(P), "i"(k)); \
     if ((k) == 0) g.phase[7]++; else g.phase[slot_[k]] += now_ - g.phase_t0; g.phase_t0 = now_; } while (0)
 #else
 #define FM(k) do { } while (0)
