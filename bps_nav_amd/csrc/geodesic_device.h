@@ -101,6 +101,13 @@ BPSX_DEV void wlane2(uint32_t& a, uint32_t va, uint32_t& b, uint32_t vb, int lan
 }
 
 // lanes 8..15 of each row of 16 take src of the lane 8 below them, lanes 0..7 keep low
+// min(v, v of the lane that the DPP control names); lanes without such a lane, or outside the
+// row mask (one bit per 16 lanes), keep v.  (The other lane's value defaults to the identity of
+// the minimum, which lets the compiler fold the lane move into the v_min itself.)
+template <int Ctrl, int RowMask> BPSX_DEV uint32_t umin_dpp(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)v, Ctrl, RowMask, 0xf, false);
+  return o < v ? o : v;
+}
 BPSX_DEV float lanes_up8(float low, float src) {
   return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(low), __float_as_int(src), 0x118 /* row_shr:8 */, 0xf, 0xf, false));
 }
@@ -339,7 +346,7 @@ struct OpenList {
     if (P == 1) {
       // No branches: without an old entry its place is -1, as an unsigned bound that keeps every lane
       const unsigned long long g0 = lanes_where(t[0] > t_), h0 = lanes_where(n[0] == n_);
-      const unsigned long long m0 = g0 & lanes_where((uint32_t)lane <= (uint32_t)first_lane(h0));
+      const unsigned long long m0 = g0 & (h0 | (h0 - 1ull));   // the lanes up to the old entry's; without one, all
       const int p = first_lane(m0);   // never empty: the unused places compare greater
       t[0] = pick(m0, from_below(t[0]), t[0]);
       n[0] = pick(m0, from_below(n[0]), n[0]);
@@ -1048,7 +1055,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     const uint32_t ip = cand >> 11;
     const unsigned long long goal = lanes_where(ip == endIp) & kRowStart;
     bool pairTie = false, goalInPair = false;
-    unsigned long long rowsAt1 = kRows1;   // rows whose updates must lie above entry 1's total
     if (__builtin_expect((goal | ((uniq & 1ull) ^ 1ull) | resolved) != 0, 0)) {
       if (resolved) { lim = 1; resolved = 0; }   // the caller has put the reference's next node first
       else if (lim == 0) {
@@ -1060,7 +1066,6 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
         if (!(uniq & 2ull)) return kAstarTie;
         pairTie = true;
         g.pairTies++;   // counts the attempts: one that fails comes back through the log
-        rowsAt1 = kRows2;
         lim = __builtin_ctzll(~(uniq | 3ull) | (1ull << kRows));
       }
       if ((goal & 1ull) && !pairTie) {
@@ -1152,13 +1157,21 @@ BPSX_DEV AstarExit astar_fast(GeoWave& g, AstarState& st, const AEdge* edges, ui
     int c = lim;
     bool pairFails = false;
     if (lim > 1) {
-      // the first entry j that an update of a row before it reaches or undercuts
-      int jv = kRows;
-#pragma unroll
-      for (int j = kRows - 1; j >= 1; --j) {
-        const unsigned long long v = lanes_where(tb <= rlane(ol.t[0], j)) & (j == 1 ? rowsAt1 : rows_below(j));
-        jv = v ? j : jv;
-      }
+      // the first entry j that an update of a row before it reaches or undercuts: the smallest
+      // updated total of every row, then of all rows up to it (a scan over the rows), and entry j's
+      // lane compares its total with that of the rows before j
+      uint32_t low = tb;   // all ones where the lane updates nothing
+      low = umin_dpp<0xb1, 0xf>(low);    // quad_perm [1,0,3,2]
+      low = umin_dpp<0x4e, 0xf>(low);    // quad_perm [2,3,0,1]
+      low = umin_dpp<0x141, 0xf>(low);   // row_half_mirror: every lane has its row's smallest
+      low = umin_dpp<0x118, 0xf>(low);   // row_shr:8: odd rows, with the row before
+      low = umin_dpp<0x142, 0xa>(low);   // row_bcast:15 into the second and fourth 16 lanes
+      low = umin_dpp<0x143, 0xc>(low);   // row_bcast:31 into the upper 32 lanes
+      uint32_t before = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - 1) * (kRowLanes * 4), (int)low);
+      // a tied pair: both its rows must lie above entry 1's total
+      if (__builtin_expect(pairTie, 0)) before = lane == 1 ? rlane(low, kRowLanes) : before;
+      const unsigned long long reached = lanes_where(before <= ol.t[0]) & (rows_below(1) & ~1ull);
+      const int jv = reached ? __builtin_ctzll(reached) : kRows;
       c = jv < c ? jv : c;
       // conflicts: the earliest row that updates a polygon leaves its mark (pass, row) at the
       // polygon's hash, later rows look for it: a mark of this pass is base + row
